@@ -138,7 +138,8 @@ class CacheManager:
     def commit(self, request, total_tokens: int) -> None:
         """Tokens [0, total_tokens) are now cached.  Window groups give back
         the pages that no later query can see: a query at p >= total sees keys
-        r > p - W, so a page whose last token is <= total - W is dead."""
+        r > p - W, so a page whose last token is <= total - W is dead, unless it
+        holds one of the first ``keep_first`` tokens, which every query sees."""
         self.lengths[request] = total_tokens
         bs = self.page_size
         for g in self.page_groups:
@@ -146,7 +147,8 @@ class CacheManager:
                 continue
             table = g.tables[request]
             dead_pages = max(0, (total_tokens - g.window + 1) // bs)
-            for j in range(min(dead_pages, len(table))):
+            kept_pages = -(-g.spec.keep_first // bs)
+            for j in range(kept_pages, min(dead_pages, len(table))):
                 if table[j] != RELEASED:
                     g.allocator.give([table[j]])
                     table[j] = RELEASED

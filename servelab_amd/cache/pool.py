@@ -5,7 +5,8 @@ Reference: ``KVCachePool`` keeps ``k_store``/``v_store`` of shape
 never cleared on reuse (servelab/kv_cache/pool.py:49-57).  Here each page group
 has one allocation per side, laid out for the attention kernels:
     k [streams, pages, nkv, page_size, D]   (a key is contiguous over D)
-    v [streams, pages, nkv, D, page_size]   (a channel is contiguous over the page)
+    v [streams, pages, nkv, Dv, page_size]  (a channel is contiguous over the page; Dv = D
+                                             unless the need says otherwise, 0 for none)
 and each state group has [streams, slots, *shape].  Storage dtype is the
 activation dtype, so a float32 model keeps a float32 cache
 (servelab/kv_cache/pool.py:41-45).
@@ -49,7 +50,7 @@ class CachePool:
             self.k.append(torch.zeros(len(g.streams), manager.num_pages, s.num_kv_heads, bs,
                                       s.head_dim, dtype=act_dtype, device=device))
             self.v.append(torch.zeros(len(g.streams), manager.num_pages, s.num_kv_heads,
-                                      s.head_dim, bs, dtype=act_dtype, device=device))
+                                      s.v_dim, bs, dtype=act_dtype, device=device))
         for g in manager.state_groups:
             self.state.append(torch.zeros(len(g.streams), manager.state_slots.num_slots,
                                           *g.spec.shape, dtype=_STATE_DTYPES[g.spec.dtype],
@@ -73,5 +74,5 @@ class CachePool:
         total = 0
         for spec in stream_specs.values():
             if hasattr(spec, "num_kv_heads"):
-                total += 2 * spec.num_kv_heads * spec.head_dim * page_size * itemsize
+                total += spec.num_kv_heads * (spec.head_dim + spec.v_dim) * page_size * itemsize
         return total

@@ -1,4 +1,6 @@
 from .model import ConfigError, Qwen2Config, read_key
+from .layered import (BiasedAttentionConfig, DenseMlpConfig, LatentAttentionConfig, LayerConfig,
+                      TopelornConfig, WindowConfig)
 from .engine import CacheConfig, SchedulerConfig, EngineConfig, PAGE_SIZES
 from .registry import (Architecture, register_architecture, registered_architectures,
                        resolve_architecture)

@@ -4,7 +4,7 @@ model builder.
 The reference has no registry: it checks ``model_type`` against a tuple
 (servelab/config.py:50-54) and looks the q/k/v bias up by architecture
 (servelab/parallel/tp_model.py:29).  Here config.json's ``architectures[0]``
-(falling back to ``model_type``) selects an entry; the entry's configuration
+(or its ``architecture`` string, falling back to ``model_type``) selects an entry; the entry's configuration
 class reads config.json and its builder turns that configuration into a
 ``ModelSpec`` (servelab_amd/parts/model.py) made of parts.
 """
@@ -37,6 +37,8 @@ def registered_architectures():
 
 def resolve_architecture(cfg: Dict[str, Any]) -> Architecture:
     archs = cfg.get("architectures") or []
+    if not archs and isinstance(cfg.get("architecture"), str):
+        archs = [cfg["architecture"]]           # designs whose config.json names one architecture
     name = archs[0] if archs else _MODEL_TYPES.get(cfg.get("model_type", ""), None)
     if name is None or name not in _ARCHITECTURES:
         asked = archs[0] if archs else f"model_type={cfg.get('model_type')!r}"

@@ -1,0 +1,79 @@
+// Products with one small matrix per head:  y[t, h, :] = A[h] x[t, h, :]
+// for all tokens t and heads h, A [heads][N][K] in the activation type, sums in
+// float.  x and y are addressed by a row stride and a head stride, so the
+// operands may be columns of wider buffers.  This is what a mixer needs whose
+// keys and values are made per head from a shared low-rank latent: the query
+// is taken to the latent's space (A[h] = Wuk[h]^T) and the attention's output
+// back from it (A[h] = Wuv[h]).
+//
+// A workgroup owns 64 tokens x 64 outputs of one head; K goes through LDS in
+// chunks of 16, every thread keeps 4 x 4 sums.
+#include "common.h"
+
+constexpr int HG_TILE = 64;
+constexpr int HG_CHUNK = 16;
+
+__global__ __launch_bounds__(256) void head_products_kernel(
+    const act_t* __restrict__ x, long long x_row, int x_head, const act_t* __restrict__ A,
+    act_t* __restrict__ y, long long y_row, int y_head, int T, int N, int K) {
+  __shared__ float xs[HG_CHUNK][HG_TILE + 1];
+  __shared__ float as[HG_CHUNK][HG_TILE + 1];
+  const int h = blockIdx.z, n0 = blockIdx.x * HG_TILE, t0 = blockIdx.y * HG_TILE;
+  const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+  const act_t* xh = x + (size_t)h * x_head;
+  const act_t* Ah = A + (size_t)h * N * K;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += HG_CHUNK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + i * 256, r = idx / HG_CHUNK, kk = idx % HG_CHUNK;
+      const int k = k0 + kk;
+      xs[kk][r] = (t0 + r < T && k < K) ? to_f(xh[(size_t)(t0 + r) * x_row + k]) : 0.f;
+      as[kk][r] = (n0 + r < N && k < K) ? to_f(Ah[(size_t)(n0 + r) * K + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < HG_CHUNK; ++kk) {
+      float xv[4], av[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) xv[i] = xs[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) av[j] = as[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += xv[i] * av[j];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = t0 + ty * 4 + i;
+    if (t >= T) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < N) y[(size_t)t * y_row + (size_t)h * y_head + n] = from_f<act_t>(acc[i][j]);
+    }
+  }
+}
+
+extern "C" const char* sl_head_products(const void* x, long long x_row, int x_head, const void* A,
+                                        void* y, long long y_row, int y_head, int T, int heads, int N,
+                                        int K, hipStream_t stream) {
+  SL_CHECK(T >= 0 && heads > 0 && N > 0 && K > 0, "head_products: sizes must be positive");
+  SL_CHECK(heads <= 65535, "head_products: more than 65535 heads");
+  SL_CHECK(x_head >= K && y_head >= N, "head_products: heads overlap");
+  SL_CHECK(x_row >= (long long)(heads - 1) * x_head + K && y_row >= (long long)(heads - 1) * y_head + N,
+           "head_products: rows are shorter than their heads");
+  if (T == 0) return nullptr;
+  const dim3 grid((N + HG_TILE - 1) / HG_TILE, (T + HG_TILE - 1) / HG_TILE, heads);
+  SL_CHECK(grid.y <= 65535, "head_products: too many rows");
+  head_products_kernel<<<grid, 256, 0, stream>>>((const act_t*)x, x_row, x_head, (const act_t*)A,
+                                                 (act_t*)y, y_row, y_head, T, N, K);
+  return sl_launch_status();
+}

@@ -156,3 +156,72 @@ extern "C" const char* sl_add_rmsnorm(float* resid, const void* delta, const flo
                                                 (act_t*)out, H, eps);
   return sl_launch_status();
 }
+
+// Layer norm with a gain and no bias, fused with the residual add that precedes it:
+//   resid (float, in place) += d1 + d2;  out = (resid - mean) / sqrt(var + eps) * w
+// where var is the mean of the squared deviations.  Either delta may be absent.
+// rows as above: with rows the stream is only read.  One block per row; the
+// row is read three times (sum, squared deviations, output), from cache after
+// the first.
+__global__ void add_layernorm_kernel(float* __restrict__ resid, const act_t* __restrict__ d1,
+                                     const act_t* __restrict__ d2, const int* __restrict__ rows,
+                                     const float* __restrict__ w, act_t* __restrict__ out, int H,
+                                     float eps) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t src = rows != nullptr ? (size_t)rows[r] : (size_t)r;
+  float* x = resid + src * H;
+  const act_t* a = d1 != nullptr ? d1 + src * H : nullptr;
+  const act_t* b = d2 != nullptr ? d2 + src * H : nullptr;
+  const bool adds = a != nullptr || b != nullptr;
+  const bool again = adds && rows != nullptr;        // the sum is not stored: form it on every pass
+  auto value = [&](int i) {
+    float d = 0.f;
+    if (a != nullptr) d = to_f(a[i]);
+    if (b != nullptr) d += to_f(b[i]);
+    return x[i] + d;
+  };
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = x[i];
+    if (adds) {
+      v = value(i);
+      if (rows == nullptr) x[i] = v;
+    }
+    sum += v;
+  }
+  const float mean = block_sum(sum, scratch) / (float)H;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float dv = (again ? value(i) : x[i]) - mean;
+    sq += dv * dv;
+  }
+  const float inv = 1.f / sqrtf(block_sum(sq, scratch) / (float)H + eps);
+  act_t* o = out + (size_t)r * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    o[i] = from_f<act_t>(((again ? value(i) : x[i]) - mean) * inv * w[i]);
+}
+
+extern "C" const char* sl_add_layernorm(float* resid, const void* d1, const void* d2, const int* rows,
+                                        const float* w, void* out, int R, int H, float eps,
+                                        hipStream_t stream) {
+  SL_CHECK(R >= 0 && H > 0, "add_layernorm: sizes must be positive");
+  if (R == 0) return nullptr;
+  const int threads = H >= 2048 ? 512 : 256;
+  add_layernorm_kernel<<<R, threads, 0, stream>>>(resid, (const act_t*)d1, (const act_t*)d2, rows, w,
+                                                  (act_t*)out, H, eps);
+  return sl_launch_status();
+}
+
+// resid (float, in place) += delta: for a delta that a norm cannot take with its own add.
+__global__ void add_into_kernel(float* __restrict__ resid, const act_t* __restrict__ delta, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) resid[i] += to_f(delta[i]);
+}
+
+extern "C" const char* sl_add_into(float* resid, const void* delta, long long n, hipStream_t stream) {
+  SL_CHECK(n >= 0, "add_into: the count must not be negative");
+  if (n == 0) return nullptr;
+  add_into_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(resid, (const act_t*)delta, (size_t)n);
+  return sl_launch_status();
+}

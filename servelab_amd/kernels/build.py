@@ -171,14 +171,15 @@ def load(u: Unit) -> ctypes.CDLL:
     return _loaded[u]
 
 
-# every unit the package can ask for with the default set of head sizes
+# the units every model needs; LAZY_STEMS are compiled when a model first asks for them
 DEFAULT_STEMS = ("elementwise", "norm", "gemm", "attention", "sampling")
+LAZY_STEMS = ("window_attention", "head_gemm")
 
 
 def all_units(head_dims=(32, 64, 96, 128, 192, 256)) -> List[Unit]:
     units = []
     for dtype in ("bfloat16", "float32"):
-        for stem in DEFAULT_STEMS:
+        for stem in DEFAULT_STEMS + LAZY_STEMS:
             units.append(unit(stem, dtype))
     for d in head_dims:
         if d % 32 == 0:

@@ -24,6 +24,7 @@ class NormOps:
         T, H = resid.shape
         self._check(resid, torch.float32, None, "residual stream")
         self._check(weight, torch.float32, (H,), "norm weight")
+        delta = self._fold_deltas(resid, delta)
         if isinstance(delta, Deferred):
             if fuse:
                 return self._produce_scaled_rows(resid, delta, weight, eps)
@@ -32,6 +33,16 @@ class NormOps:
         self._call("norm", "sl_add_rmsnorm", _p(resid), *self._delta_args(delta, T, H), None,
                    _p(weight), _p(out), T, H, _c_float(eps))
         return out
+
+    def _fold_deltas(self, resid, delta):
+        """A tuple of deltas (sublayers that ran side by side): all but the last are added into
+        the stream here; the last is returned for the norm's own add."""
+        if not isinstance(delta, (tuple, list)):
+            return delta
+        values = [d for d in delta if d is not None]
+        for d in values[:-1]:
+            self.add_into(resid, self.materialize(d))
+        return values[-1] if values else None
 
     def _delta_args(self, delta, T, H):
         """(delta, parts, nparts, T, bias) of the norm kernels for any kind of delta."""
@@ -53,6 +64,7 @@ class NormOps:
         self._check(resid, torch.float32, None, "residual stream")
         self._check(weight, torch.float32, (H,), "norm weight")
         self._check(rows, torch.int32, (R,), "rows")
+        delta = self._fold_deltas(resid, delta)
         if isinstance(delta, Deferred):
             if fuse and R <= self._fused_rows(H):
                 scaled = self._produce_scaled_rows(resid, delta, weight, eps)

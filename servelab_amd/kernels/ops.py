@@ -17,11 +17,13 @@ from .norm_ops import NormOps
 from .product_ops import ProductOps
 from .sampling_ops import SamplingOps
 from .table import KernelTable
+from .window_ops import WindowOps
 from .values import (Deferred, KernelError, LinearWeight, PartialSums, RotationPlan,  # noqa: F401
                      ScaledRows, TiledRows, _RopeStore, _c_float, _p, _ptr)
 
 
-class HipOps(NormOps, ProductOps, AttentionOps, SamplingOps, KernelTable):
+class HipOps(NormOps, ProductOps, AttentionOps, WindowOps, SamplingOps, KernelTable):
     """The whole table: the base (libraries, calls, checks) and one group of calls per domain.
     ``norm_ops``: embedding, add + norm, silu-multiply; ``product_ops``: weights and products;
-    ``attention_ops``: rotation, cache write, attention; ``sampling_ops``: argmax and draws."""
+    ``attention_ops``: rotation, cache write, attention; ``sampling_ops``: argmax and draws;
+    ``window_ops``: layer norm, per-head products, attention with a kept-first window, bias, sink and gate."""

@@ -22,10 +22,19 @@ class ParamSpec:
 @dataclass(frozen=True)
 class PagedKVSpec:
     """Cache need: keys and values of past tokens, in pages.  ``window`` None
-    keeps every token; a window W keeps the last W."""
+    keeps every token; a window W keeps the last W, and the first
+    ``keep_first`` tokens of the sequence besides.  ``value_dim``: channels of
+    a value (None: as many as a key's; 0: no values are stored, the mixer reads
+    them out of the key rows)."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
+    keep_first: int = 0
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else int(self.value_dim)
 
 
 @dataclass(frozen=True)

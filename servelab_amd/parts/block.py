@@ -4,6 +4,10 @@ PreNormBlock: h += Mixer(Norm1(h)); h += FeedForward(Norm2(h))
 (servelab/parallel/tp_model.py:124-133).  The adds are fused into the norm
 that follows them, so a block returns its feed-forward output as a pending
 delta for the next norm to add.
+
+ParallelBlock: with x = Norm(h), h += Mixer(x) + FeedForward(x): one norm, both
+sublayers read its output; the block returns both outputs as its pending delta
+(a tuple), which the next norm adds to the stream in float32.
 """
 from .base import Block, prefixed
 
@@ -42,3 +46,44 @@ class PreNormBlock(Block):
         a = self.mixer.forward(x, batch, caches[0] if caches else None, shared)
         x2 = self.norm2.forward(resid, a, fuse=self.feedforward.takes_scaled_rows)
         return self.feedforward.forward(x2)
+
+
+class ParallelBlock(Block):
+    """``feedforward`` may be None: the mixer alone."""
+
+    def __init__(self, norm, mixer, feedforward, names=("norm.", "mixer.", "mlp.")):
+        self.norm, self.mixer, self.feedforward = norm, mixer, feedforward
+        self.names = tuple(names)
+
+    @property
+    def graph_safe(self):
+        return all(part.graph_safe for _, part in self._children())
+
+    def _children(self):
+        parts = [(self.names[0], self.norm), (self.names[1], self.mixer)]
+        if self.feedforward is not None:
+            parts.append((self.names[2], self.feedforward))
+        return parts
+
+    def cache_specs(self):
+        spec = self.mixer.cache_spec()
+        return [] if spec is None else [spec]
+
+    def param_specs(self):
+        specs = {}
+        for prefix, part in self._children():
+            for name, spec in part.param_specs().items():
+                specs[prefix + name] = spec
+        return specs
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        for prefix, part in self._children():
+            part.load(prefixed(prefix, tensors), rt)
+
+    def forward(self, resid, delta, batch, caches, shared):
+        x = self.norm.forward(resid, delta)
+        a = self.mixer.forward(x, batch, caches[0] if caches else None, shared)
+        if self.feedforward is None:
+            return a
+        return (a, self.feedforward.forward(x))

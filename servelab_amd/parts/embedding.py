@@ -10,15 +10,16 @@ from .base import Embedding, Part, ParamSpec
 class TokenEmbedding(Embedding):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, name: str = "weight"):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.name = name
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+        return {self.name: ParamSpec((self.vocab_size, self.hidden_size))}
 
     def load(self, tensors, rt):
         self.rt = rt
-        self.weight = rt.matrix(tensors("weight"))
+        self.weight = rt.matrix(tensors(self.name))
 
     def forward(self, batch):
         """The rows of the table at ``batch.ids`` (int32 [T]) as the float32

@@ -15,21 +15,23 @@ class GatedMLP(FeedForward):
     graph_safe = True
     takes_scaled_rows = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu",
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
         if activation != "silu":
             raise ValueError(f"GatedMLP: activation '{activation}' is not supported")
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
+        self.names = tuple(names)          # checkpoint names of the gate, up and down matrices
 
     def param_specs(self):
         h, i = self.hidden_size, self.intermediate_size
-        return {"gate_proj.weight": ParamSpec((i, h)),
-                "up_proj.weight": ParamSpec((i, h)),
-                "down_proj.weight": ParamSpec((h, i))}
+        return {self.names[0]: ParamSpec((i, h)),
+                self.names[1]: ParamSpec((i, h)),
+                self.names[2]: ParamSpec((h, i))}
 
     def load(self, tensors, rt):
         self.rt = rt
-        gate, up = tensors("gate_proj.weight"), tensors("up_proj.weight")
+        gate, up = tensors(self.names[0]), tensors(self.names[1])
         i, h = self.intermediate_size, self.hidden_size
         self.block = getattr(rt.ops, "GATE_BLOCK", i)
         if i % self.block:
@@ -37,7 +39,7 @@ class GatedMLP(FeedForward):
         b = self.block
         self.w_gate_up = rt.linear_weight(torch.stack(
             [gate.reshape(i // b, b, h), up.reshape(i // b, b, h)], 1).reshape(2 * i, h))
-        self.w_down = rt.linear_weight(tensors("down_proj.weight"), delta=True)
+        self.w_down = rt.linear_weight(tensors(self.names[2]), delta=True)
 
     def forward(self, x):
         ops = self.rt.ops

@@ -1,4 +1,5 @@
-"""RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w in float32.
+"""RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w in float32; LayerNorm with a gain and
+no bias: y = (x - mean) / sqrt(var + eps) * w, var the mean of the squared deviations.
 
 Reference: servelab/attention/triton/paged_attention.py:76-91 and the vector
 in tests/test_triton_kernels.py:57-59.  Here the residual add that precedes
@@ -10,19 +11,46 @@ from .base import Norm, ParamSpec
 class RMSNorm(Norm):
     graph_safe = True
 
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, name: str = "weight"):
         self.size = int(size)
         self.eps = float(eps)
+        self.name = name
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.size,), init="gain")}
+        return {self.name: ParamSpec((self.size,), init="gain")}
 
     def load(self, tensors, rt):
         self.rt = rt
-        self.weight = rt.vector(tensors("weight"))
+        self.weight = rt.vector(tensors(self.name))
 
     def forward(self, resid, delta, fuse=False):
         return self.rt.ops.add_rmsnorm(resid, delta, self.weight, self.eps, fuse=fuse)
 
     def forward_rows(self, resid, delta, rows, fuse=False):
         return self.rt.ops.rows_add_rmsnorm(resid, delta, rows, self.weight, self.eps, fuse=fuse)
+
+
+class LayerNorm(Norm):
+    """Layer norm with a gain and no bias, in float32, fused with the residual
+    add before it.  ``delta`` may be a tuple of values that are all added (the
+    outputs of sublayers that ran side by side).  Its rows are plain normed rows
+    (``fuse`` is not taken up)."""
+    graph_safe = True
+
+    def __init__(self, size: int, eps: float, name: str = "weight"):
+        self.size = int(size)
+        self.eps = float(eps)
+        self.name = name
+
+    def param_specs(self):
+        return {self.name: ParamSpec((self.size,), init="gain")}
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        self.weight = rt.vector(tensors(self.name))
+
+    def forward(self, resid, delta, fuse=False):
+        return self.rt.ops.add_layernorm(resid, delta, self.weight, self.eps)
+
+    def forward_rows(self, resid, delta, rows, fuse=False):
+        return self.rt.ops.add_layernorm(resid, delta, self.weight, self.eps, rows=rows)
