@@ -56,6 +56,69 @@ SHAPES = {"7b": ("Qwen2.5-7B shape", QWEN25_7B), "32b": ("Qwen2.5-32B shape", QW
           "14b": ("Qwen2.5-14B shape", QWEN25_14B)}
 
 
+# Layer sizes for the design comparison (--design): a Topelorn decoder whose layers have the sizes of a
+# real model's, and the Qwen2 decoder of equal size (width, heads, head size, feed-forward, layers,
+# vocabulary, the same window on every layer), both with random weights.
+DESIGN_SHAPES = {
+    "3b": dict(width=2048, heads=16, kv_heads=2, dim=128, ff=11008, vocab=32000),
+    "7b": dict(width=3584, heads=28, kv_heads=4, dim=128, ff=18944, vocab=32000),
+}
+
+
+def design_configs(shape, layers, window, keep_first=4, kv_rank=512, rot_dim=64):
+    """(Topelorn config.json, Qwen2 config.json) of equal size: every fourth Topelorn layer is a latent
+    attention, the others are attentions with a kept-first window, a sink, value mixing and a gate."""
+    z = DESIGN_SHAPES[shape]
+    attn = {"type": "attention", "mlp": {"kind": "dense", "ff": z["ff"]},
+            "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                      "scale": z["dim"] ** -0.5, "mask": {"size": window, "keep_first": keep_first},
+                      "v_mix": True}}
+    lat = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": z["ff"]},
+           "mixer": {"heads": z["heads"], "dim": z["dim"], "rot_dim": rot_dim, "vdim": z["dim"],
+                     "kv_rank": kv_rank, "scale": (z["dim"] + rot_dim) ** -0.5, "mask": {"size": window},
+                     "rot": {"base": 10000.0, "dims": rot_dim}}}
+    topelorn = {"architecture": "Topelorn", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-5},
+                "torch_dtype": "bfloat16", "layers": [lat if i % 4 == 3 else attn for i in range(layers)]}
+    qwen = dict(QWEN25_7B, num_hidden_layers=layers, hidden_size=z["width"], num_attention_heads=z["heads"],
+                num_key_value_heads=z["kv_heads"], head_dim=z["dim"], intermediate_size=z["ff"],
+                vocab_size=z["vocab"], tie_word_embeddings=True, use_sliding_window=True,
+                sliding_window=window, max_window_layers=0)
+    return topelorn, qwen
+
+
+def compare_designs(args):
+    """Prefill and decode throughput of the Topelorn design beside the Qwen2 decoder of equal size, at
+    each of --design-shapes: one JSON line, tokens per second each."""
+    import torch
+    import servelab_amd  # noqa: F401
+    from servelab_amd.config import resolve_architecture
+    from servelab_amd.engine.session import random_model_on_device
+    page = args.block_size
+    out = {"metric": "design_comparison", "unit": "tok/s", "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic: seeded random weights, uniform random token ids", "n_gpus": 1,
+           "config": {"layers": args.design_layers, "window": args.design_window, "decode_batch": args.batch,
+                      "decode_context": args.context, "prefill_tokens": args.prefill_tokens,
+                      "prefill_chunk": args.prefill_chunk, "page_size": page}, "shapes": {}}
+    for shape in args.design_shapes.split(","):
+        row = {}
+        for name, raw in zip(("topelorn", "qwen2"), design_configs(shape, args.design_layers, args.design_window)):
+            cfg = resolve_architecture(raw).config_from_hf(raw, "")
+            model = random_model_on_device(cfg, args.seed, args.dtype, "cuda:0")
+            torch.cuda.synchronize()
+            step_s, _, _ = time_decode(cfg, model, args.batch, args.context, args.steps, args.warmup, page)
+            pre_s, _ = time_prefill(model, args.prefill_tokens, page, repeats=5, max_chunk=args.prefill_chunk,
+                                    tune=not args.no_tune)
+            row[name] = {"decode_tok_s": round(args.batch / step_s, 1), "decode_ms_per_step": round(step_s * 1e3, 4),
+                         "prefill_tok_s": round(args.prefill_tokens / pre_s, 1), "prefill_ms": round(pre_s * 1e3, 3)}
+            del model
+            torch.cuda.empty_cache()
+        row["decode_ratio"] = round(row["topelorn"]["decode_tok_s"] / row["qwen2"]["decode_tok_s"], 3)
+        row["prefill_ratio"] = round(row["topelorn"]["prefill_tok_s"] / row["qwen2"]["prefill_tok_s"], 3)
+        out["shapes"][shape] = row
+    print(json.dumps(out))
+    return 0
+
+
 def build(args):
     import torch
     import servelab_amd  # noqa: F401
@@ -203,11 +266,19 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernel choice for the prompt products")
+    ap.add_argument("--design", default="", choices=["", "topelorn"],
+                    help="instead of the default workload: prefill and decode throughput of this design "
+                         "beside the Qwen2 decoder of equal size")
+    ap.add_argument("--design-shapes", default="3b,7b", help="comma-separated: " + ", ".join(sorted(DESIGN_SHAPES)))
+    ap.add_argument("--design-layers", type=int, default=4)
+    ap.add_argument("--design-window", type=int, default=1024)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
         return 2
 
+    if args.design:
+        return compare_designs(args)
     cfg, model, full_layers = build(args)
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     itemsize = 2 if short == "bf16" else 4

@@ -30,7 +30,7 @@ def _section(cfg: Dict[str, Any], key: str, where: str, required=True) -> Option
 
 @dataclass(frozen=True)
 class WindowConfig:
-    """Query i sees key j <= i when i - j < size or j < keep_first."""
+    """Query i sees key j <= i when i - j < size or j < keep_first; size 0: every j <= i."""
     size: int
     keep_first: int = 0
 
@@ -72,7 +72,9 @@ class LayerConfig:
 
 
 def _window(mixer: Dict[str, Any], where: str, keeps: bool) -> WindowConfig:
-    mask = _section(mixer, "mask", where)
+    mask = _section(mixer, "mask", where, required=False)
+    if mask is None:
+        return WindowConfig(0, 0)                   # no mask: every earlier key
     size = read_key(mask, "size", kind=int)
     keep = read_key(mask, "keep_first", 0, kind=int) if keeps else 0
     if size < 1 or keep < 0:
@@ -132,6 +134,19 @@ class TopelornConfig:
     path: str = ""
     raw: Dict[str, Any] = field(default_factory=dict, repr=False, compare=False)
 
+    # the names the rest of the engine reads a model's sizes by
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
+    @property
+    def hidden_size(self) -> int:
+        return self.width
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
     @classmethod
     def from_hf(cls, cfg: Dict[str, Any], path: str = "") -> "TopelornConfig":
         norm = _section(cfg, "norm", "model")
@@ -156,6 +171,8 @@ class TopelornConfig:
 
     def to_hf(self) -> Dict[str, Any]:
         def mask(w, keeps):
+            if not w.size:
+                return None
             return {"size": w.size, "keep_first": w.keep_first} if keeps else {"size": w.size}
         layers = []
         for l in self.layers:

@@ -176,6 +176,11 @@ DEFAULT_STEMS = ("elementwise", "norm", "gemm", "attention", "sampling")
 LAZY_STEMS = ("window_attention", "head_gemm")
 
 
+# (key width, value width, values in the key rows) the matrix-core window attention is built for
+# ahead of use; other widths are compiled when a model first needs them
+WINDOW_MFMA_SIZES = ((128, 128, 0), (64, 64, 0), (576, 512, 1), (32, 16, 0), (64, 48, 1), (96, 64, 0))
+
+
 def all_units(head_dims=(32, 64, 96, 128, 192, 256)) -> List[Unit]:
     units = []
     for dtype in ("bfloat16", "float32"):
@@ -184,4 +189,6 @@ def all_units(head_dims=(32, 64, 96, 128, 192, 256)) -> List[Unit]:
     for d in head_dims:
         if d % 32 == 0:
             units.append(unit("attention_mfma", "bfloat16", SL_HEAD_DIM=d))
+    for dk, dv, vk in WINDOW_MFMA_SIZES:
+        units.append(unit("window_attention_mfma", "bfloat16", SL_DK=dk, SL_DV=dv, SL_VK=vk))
     return units

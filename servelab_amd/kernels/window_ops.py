@@ -14,8 +14,31 @@ _ll = ctypes.c_longlong
 
 class WindowOps:
     # shares of the keys for steps of single tokens: one share per this many keys a token sees
+    # (the float kernel, the matrix-core kernel)
     WINDOW_SHARE_KEYS = 256
     WINDOW_MAX_SHARES = 16
+    WINDOW_MFMA_SHARE_KEYS = 128
+    WINDOW_MFMA_MAX_SHARES = 32
+    WINDOW_MFMA_LDS_BYTES = 160 * 1024
+
+    def _window_mfma_fits(self, q, q_col, Dk, Dv):
+        """The matrix-core kernel takes bfloat16, key widths in steps of 32 and value widths in steps
+        of 16 whose staged block fits LDS, and q rows that are 16-byte aligned; everything else goes
+        to the float kernel."""
+        if self.act_dtype != torch.bfloat16 or not self.use_mfma_attention:
+            return False
+        if Dk % 32 or Dv % 16 or Dk > 1024 or Dv > 512:
+            return False
+        if 2 * (32 * (Dk + 8) + Dv * 40) > self.WINDOW_MFMA_LDS_BYTES:
+            return False
+        return q.shape[1] % 8 == 0 and q_col % 8 == 0 and q.data_ptr() % 16 == 0
+
+    def _window_mfma_lib(self, Dk, Dv, in_keys):
+        key = ("window_attention_mfma", Dk, Dv, in_keys)
+        if key not in self._lib:
+            self._lib[key] = build.load(build.unit("window_attention_mfma", "bfloat16", SL_DK=Dk, SL_DV=Dv,
+                                                   SL_VK=int(in_keys)))
+        return key
 
     def _lazy(self, stem):
         """The library of ``stem`` for this table's dtype, compiled and loaded at first use."""
@@ -181,18 +204,28 @@ class WindowOps:
         window = int(window or 0)
         # shares of the keys: for steps of single tokens only (a prompt's tiles are many), by the
         # number of keys a token can see there; fixed by sizes that a captured step keeps
+        mfma = self._window_mfma_fits(q, q_col, Dk, Dv)
         nsplit = 1
         if batch.max_q_len == 1:
             span = batch.max_ctx_len if not window else min(batch.max_ctx_len, window + int(keep_first))
-            nsplit = max(1, min(self.WINDOW_MAX_SHARES, span // self.WINDOW_SHARE_KEYS))
+            nsplit = max(1, min(self.WINDOW_MFMA_MAX_SHARES, span // self.WINDOW_MFMA_SHARE_KEYS) if mfma
+                         else min(self.WINDOW_MAX_SHARES, span // self.WINDOW_SHARE_KEYS))
         part_o = part_ml = None
         if nsplit > 1:
             part_o = self._new((T, nh, nsplit, Dv), torch.float32)
             part_ml = self._new((T, nh, nsplit, 2), torch.float32)
         out = self._new((T, nh * Dv))
         item = q.element_size()
-        lib = self._lazy("window_attention")
-        self._call(lib, "sl_window_attention", _c_void_p(q.data_ptr() + q_col * item), q.shape[1], _p(k_cache),
+        if mfma:
+            lib = self._window_mfma_lib(Dk, Dv, v_cache is None)
+            name = f"sl_window_attention_mfma@{Dk}.{Dv}.{int(v_cache is None)}"
+            if name not in self._fn:
+                fn = self._lib[lib].sl_window_attention_mfma
+                fn.restype = ctypes.c_char_p
+                self._fn[name] = fn
+        else:
+            lib, name = self._lazy("window_attention"), "sl_window_attention"
+        self._call(lib, name, _c_void_p(q.data_ptr() + q_col * item), q.shape[1], _p(k_cache),
                    _p(v_cache), _p(block_tables), max_pages, _p(batch.cu_q), _p(batch.positions),
                    S, batch.max_q_len, T, nh, nkv, Dk, Dv, page_size, _c_float(scale), window,
                    int(keep_first), _p(slopes), _p(sinks),

@@ -28,6 +28,14 @@ import torch
 
 from .base import Mixer, PagedKVSpec, ParamSpec
 
+def _padded_rows(rows):
+    """[rows...] concatenated, with zero rows added up to a multiple of 8: the product's output
+    rows then start 16-byte aligned in both activation types."""
+    w = torch.cat(rows, 0)
+    extra = -w.shape[0] % 8
+    return torch.cat([w, w.new_zeros(extra, w.shape[1])], 0) if extra else w
+
+
 _WINDOW_NAMES = {"q": "q", "k": "k", "v": "v", "q_norm": "q.norm", "k_norm": "k.norm",
                  "mix": "vmix", "sink": "sink", "gate": "g", "out": "o"}
 
@@ -86,7 +94,7 @@ class GatedWindowAttention(Mixer):
         rows = [tensors(n["q"]), tensors(n["k"]), tensors(n["v"])]
         if self.gate:
             rows.append(tensors(n["gate"]))
-        self.w_in = rt.linear_weight(torch.cat(rows, 0))          # [q; k; v; gate] in one product
+        self.w_in = rt.linear_weight(_padded_rows(rows))          # [q; k; v; gate] in one product
         self.w_o = rt.linear_weight(tensors(n["out"]), delta=True)
         self.q_gain = rt.vector(tensors(n["q_norm"])) if self.qk_norm else None
         self.k_gain = rt.vector(tensors(n["k_norm"])) if self.qk_norm else None
@@ -170,7 +178,7 @@ class LatentWindowAttention(Mixer):
         rows = [tensors(n["q"]), tensors(n["down"])]
         if self.gate:
             rows.append(tensors(n["gate"]))
-        self.w_in = rt.linear_weight(torch.cat(rows, 0))          # [q; down; gate] in one product
+        self.w_in = rt.linear_weight(_padded_rows(rows))          # [q; down; gate] in one product
         self.w_o = rt.linear_weight(tensors(n["out"]), delta=True)
         self.gain = rt.vector(tensors(n["down_norm"]))
         # per head: Wuk_h^T [C, D] takes q to the latent's space, Wuv_h [Dv, C] brings the output back

@@ -143,3 +143,15 @@ def test_greedy_generation_through_the_entry_point(tmp_path, which, dtype):
             for i, t in enumerate(toks):
                 row = logits[len(p) - 1 + i]
                 assert row[t] >= row.max() - slack, f"token {i}: {float(row[t])} vs best {float(row.max())}"
+
+
+def test_command_line_samples_from_a_random_model(tmp_path, capsys):
+    """bin/run_engine's entry with this design's config.json, seeded random weights made on the device,
+    and a temperature with top-k and top-p cuts."""
+    import json
+    from servelab_amd import cli
+    path = tmp_path / "config.json"
+    path.write_text(json.dumps(MODELS["B"]))
+    assert cli.main(["--config", str(path), "--random-weights", "3", "--prompt-ids", "5,6,7,8", "--max-tokens", "9",
+                     "--temperature", "0.8", "--top-k", "20", "--top-p", "0.9", "--max-num-seqs", "4"]) == 0
+    assert "finish=length" in capsys.readouterr().out

@@ -153,7 +153,8 @@ def run_attention(ops, seqs, page, H, G, Dk, Dv, scale, window, keep, slopes, si
 
 
 @pytest.mark.parametrize("page", [16, 32])
-@pytest.mark.parametrize("H,G,Dk,Dv", [(4, 2, 24, 16), (3, 3, 40, 8), (6, 1, 16, 40), (20, 1, 12, 36)])
+@pytest.mark.parametrize("H,G,Dk,Dv", [(4, 2, 24, 16), (3, 3, 40, 8), (6, 1, 16, 40), (20, 1, 12, 36),
+                                       (4, 2, 32, 16), (6, 1, 96, 64), (8, 8, 64, 64)])
 def test_window_attention_prompts_and_single_tokens(ops, page, H, G, Dk, Dv):
     slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)])
     sinks = torch.randn(H, generator=torch.Generator().manual_seed(H))
@@ -168,7 +169,7 @@ def test_window_attention_prompts_and_single_tokens(ops, page, H, G, Dk, Dv):
 
 
 def test_window_attention_without_extras_and_values_from_key_rows(ops):
-    for in_keys, Dk, Dv in ((True, 48, 40), (True, 16, 16), (False, 8, 24)):
+    for in_keys, Dk, Dv in ((True, 48, 40), (True, 16, 16), (False, 8, 24), (True, 64, 48)):
         got, want = run_attention(ops, [(0, 40), (37, 5), (52, 1)], 16, 5, 1, Dk, Dv, 0.3, 13, 0, None, None,
                                   False, in_keys, seed=Dk)
         close(got, want, ops.act_dtype, scale=2.0)
@@ -177,21 +178,24 @@ def test_window_attention_without_extras_and_values_from_key_rows(ops):
 def test_single_tokens_in_shares_of_their_keys(ops):
     """Contexts long enough that a step of single tokens cuts its keys into shares, with sequences so
     short that some shares are empty."""
-    H, G, Dk, Dv = 4, 2, 16, 24
+    H, G = 4, 2
     sinks = torch.tensor([0.5, -1.0, 2.0, 0.0])
     slopes = torch.tensor([0.5, 0.25, 0.1, 0.01])
     seqs = [(1500, 1), (3, 1), (0, 1), (700, 1)]
-    for window, keep in ((None, 0), (1000, 5), (600, 40)):
-        got, want = run_attention(ops, seqs, 16, H, G, Dk, Dv, 0.25, window, keep, slopes, sinks, True, False, seed=9)
-        close(got, want, ops.act_dtype, scale=2.0)
+    for Dk, Dv in ((16, 24), (32, 16)):
+        for window, keep in ((None, 0), (1000, 5), (600, 40)):
+            got, want = run_attention(ops, seqs, 16, H, G, Dk, Dv, 0.25, window, keep, slopes, sinks, True, False,
+                                      seed=9)
+            close(got, want, ops.act_dtype, scale=2.0)
 
 
-def test_one_far_key_shows(ops):
+@pytest.mark.parametrize("Dk,Dv", [(16, 8), (32, 16)])
+def test_one_far_key_shows(ops, Dk, Dv):
     """One key is made to stand out for one query; the output is its value exactly when the window or the
     kept first tokens let it be seen.  Keys just inside and just outside, at page borders."""
     dt = ops.act_dtype
     H = G = 1
-    Dk, Dv, page, W, keep = 16, 8, 16, 48, 5
+    page, W, keep = 16, 48, 5
     for q_at, key_at, seen in ((200, 153, True), (200, 152, False), (200, 4, True), (200, 5, False),
                                (63, 16, True), (64, 16, False), (47, 0, True), (300, 0, True), (175, 128, True),
                                (176, 128, False), (176, 127, False)):

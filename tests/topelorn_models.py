@@ -53,7 +53,13 @@ MODEL_C = config(96, 128, 1e-5, [
     attention(8, 4, 32, 32, 6, 2, True, 128),
     latent(4, 24, 8, 40, 32, 7, 64),
 ])
-MODELS = {"A": MODEL_A, "B": MODEL_B, "C": MODEL_C}
+# widths the matrix-core attention takes in bfloat16 (keys in steps of 32, values in steps of 16)
+MODEL_D = config(64, 211, 1e-5, [
+    attention(4, 2, 32, 16, 9, 3, True, 96),
+    latent(3, 16, 16, 24, 48, 13, 0),
+    attention(4, 2, 32, 16, 40, 0, True, 64),
+])
+MODELS = {"A": MODEL_A, "B": MODEL_B, "C": MODEL_C, "D": MODEL_D}
 
 
 def tensor_shapes(cfg):
