@@ -11,15 +11,18 @@
 // on float accumulators.
 //
 // Work layout.  A column is a (token, query head) pair of one sequence and one kv head; a
-// wavefront owns 16 columns, a workgroup of NW wavefronts 16 NW consecutive ones, and walks the
+// wavefront owns 16 columns, a workgroup of four wavefronts 64 consecutive ones, and walks the
 // blocks of 32 keys any of them sees.  A block is staged in LDS once for the workgroup: the key
 // rows [32][SL_DK], and the values channel-major [SL_DV][32] (copied from the value pages, which
-// are channel-major already, or scattered from the key rows).  Per block and wavefront:
+// are channel-major already, or turned in registers, 8 keys x 8 channels a thread, on their way
+// from the key rows); the next block is on its way from the pages to registers while a block is
+// computed.  Per block and wavefront:
 //   S^T[key, column] = K[key, :] . Q[column, :]          mfma 16x16x32, A = K rows, B = Q (registers)
 //   O^T[d, column] += V^T[d, key] P^T[key, column]       mfma 16x16x32, A = V^T rows, B = the terms of P
 // Row i of score tile m is key 8 (i / 4) + 4 m + i % 4 of the block, so that a lane ends up with
 // the weights of 8 consecutive keys of its column: the B operand of the second product as it is.
-// Steps of single tokens run with NW = 1 and cut the blocks into shares over workgroups.
+// A step of single tokens has few columns (the heads of a group): its blocks are cut into shares
+// over workgroups, whose wavefronts without a column only help to stage.
 #include "window_attention.h"
 
 #if defined(SL_F32)
@@ -46,21 +49,36 @@ constexpr int KROW = DK + 8;          // elements of a staged key row (the pad s
 constexpr int VROW = 40;              // elements of a staged channel row: 32 keys and a pad
 constexpr float LOG2E = 1.4426950408889634f;
 
-__device__ __forceinline__ float column_max4(float x) {      // over lanes n, n + 16, n + 32, n + 48
-  x = fmaxf(x, __shfl_xor(x, 16, 64));
-  return fmaxf(x, __shfl_xor(x, 32, 64));
+// Maximum / sum over the four lanes n, n + 16, n + 32, n + 48 that share a column, by the row-swap
+// instructions of gfx950 (register to register): after a swap of x with itself one result holds
+// the lower partner and the other the upper one, in every lane.
+__device__ __forceinline__ float column_max4(float x) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float column_sum4(float x) {
-  x += __shfl_xor(x, 16, 64);
-  return x + __shfl_xor(x, 32, 64);
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-template <int NW>
-__global__ __launch_bounds__(64 * NW) void window_attention_mfma_kernel(const WindowAttention a) {
+constexpr int THREADS = 256, COLS = 64;
+constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
+// what a thread stages of a block: chunks of 8 values (16 bytes)
+constexpr int KCH = DK / 8;                            // chunks of a key row
+constexpr int NKC = VK ? 1 : cdiv(32 * KCH, THREADS);  // key chunks a thread
+constexpr int NVC = VK ? 1 : cdiv(DV * 4, THREADS);    // value chunks (a channel's 8 keys) a thread
+constexpr int RCH = VK ? (DK - DV) / 8 : 0;            // chunks of a key row behind the values
+constexpr int NT = VK ? cdiv((DV / 8) * 4, THREADS) : 1;   // 8 keys x 8 channels tiles a thread (turned on their way into LDS)
+constexpr int NR = VK ? (RCH ? cdiv(32 * RCH, THREADS) : 1) : 1;
+
+__global__ __launch_bounds__(THREADS) void window_attention_mfma_kernel(const WindowAttention a) {
   extern __shared__ __attribute__((aligned(16))) __bf16 lds16[];
   __bf16* ks = lds16;                                  // [32][KROW]
   __bf16* vt = ks + 32 * KROW;                         // [DV][VROW]
-  constexpr int THREADS = 64 * NW, COLS = 16 * NW;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, gq = lane >> 4;
   const int page = a.page, nkv = a.nkv;
   const int seq = blockIdx.z, kvh = blockIdx.y;
@@ -87,14 +105,23 @@ __global__ __launch_bounds__(64 * NW) void window_attention_mfma_kernel(const Wi
   const int nblk = nA + nB;
   const int i0 = (int)((long long)nblk * share / a.nsplit);
   const int i1 = (int)((long long)nblk * (share + 1) / a.nsplit);
+  auto block_base = [&](int i) { return (i < nA ? i : firstB + (i - nA)) * 32; };
+  auto loadable = [&](int key) { return key <= kmax && (key >= kmin || key < keep); };
 
-  // this lane's column (a column past the last is computed like the last and never stored)
-  int c = c0 + 16 * wave + n;
+  // this wavefront's columns, and this lane's (a column past the last is computed like the last, never stored)
+  const int cw0 = c0 + 16 * wave;
+  const bool wave_live = cw0 < ncols;
+  const int cw1 = cw0 + 15 < ncols - 1 ? cw0 + 15 : ncols - 1;
+  int c = cw0 + n;
   const bool live = c < ncols;
   if (!live) c = ncols - 1;
   const int tok = c / g, head = kvh * g + c % g;
   const int pos_c = pos0 + tok;
   const int lo_c = a.window > 0 && pos_c - a.window + 1 > 0 ? pos_c - a.window + 1 : 0;
+  // every column of the wavefront sees all of a block [kb, kb + 31] when kb + 31 <= pos_lo and (kb >= lo_hi
+  // or the block lies within the kept first tokens)
+  const int pos_lo = pos0 + (wave_live ? cw0 : 0) / g, pos_hi = pos0 + (wave_live ? cw1 : 0) / g;
+  const int lo_hi = a.window > 0 && pos_hi - a.window + 1 > 0 ? pos_hi - a.window + 1 : 0;
   const float scale2 = a.scale * LOG2E;
   const float slope2 = a.slopes != nullptr ? a.slopes[head] * LOG2E : 0.f;
   bf16x8 qf[KK];
@@ -110,39 +137,103 @@ __global__ __launch_bounds__(64 * NW) void window_attention_mfma_kernel(const Wi
   const __bf16 zero = (__bf16)0.f;
   const bf16x8 zeros = {zero, zero, zero, zero, zero, zero, zero, zero};
 
-  for (int i = i0; i < i1; ++i) {
-    const int kbase = (i < nA ? i : firstB + (i - nA)) * 32;
-    __syncthreads();                                   // the last block's readers are done
-    for (int idx = tid; idx < 32 * (DK / 8); idx += THREADS) {
-      const int kl = idx / (DK / 8), c8 = idx % (DK / 8), key = kbase + kl;
-      bf16x8 v = zeros;
-      if (key <= kmax && (key >= kmin || key < keep)) {
-        const int pg = table[key / page];
-        v = *(const bf16x8*)(a.kc + (((size_t)pg * nkv + kvh) * page + key % page) * DK + 8 * c8);
-      }
-      *(bf16x8*)(ks + kl * KROW + 8 * c8) = v;
-      if (VK && 8 * c8 < DV) {
+  // A block travels pages -> registers -> LDS; the registers are filled for block i + 1 while block i
+  // is computed from LDS.
+  bf16x8 kreg[NKC], vreg[NVC], treg[NT][8], rreg[NR];
+  auto fetch = [&](int kbase) {
+    const int pgA = table[kbase / page];
+    const int pgB = kbase + 16 <= kmax ? table[(kbase + 16) / page] : pgA;
+    auto key_row = [&](int kl) {                       // start of the cache row of key kbase + kl
+      const int pg = kl < 16 ? pgA : pgB;
+      return a.kc + (((size_t)pg * nkv + kvh) * page + ((kbase + kl) & (page - 1))) * DK;
+    };
+    if constexpr (!VK) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) vt[(8 * c8 + e) * VROW + kl] = v[e];
+      for (int i = 0; i < NKC; ++i) {
+        const int idx = tid + THREADS * i, kl = idx / KCH, c8 = idx % KCH;
+        kreg[i] = zeros;
+        if (idx < 32 * KCH && loadable(kbase + kl)) kreg[i] = *(const bf16x8*)(key_row(kl) + 8 * c8);
+      }
+#pragma unroll
+      for (int i = 0; i < NVC; ++i) {
+        const int idx = tid + THREADS * i, d = idx / 4, k8 = idx % 4, key0 = kbase + 8 * k8;
+        vreg[i] = zeros;
+        if (idx < DV * 4 && key0 <= kmax && (key0 + 7 >= kmin || key0 < keep)) {
+          const int pg = k8 < 2 ? pgA : pgB;
+          bf16x8 v = *(const bf16x8*)(a.vc + (((size_t)pg * nkv + kvh) * DV + d) * page + (key0 & (page - 1)));
+#pragma unroll
+          for (int e = 0; e < 8; ++e)                  // a slot of the page that holds no visible key may hold anything
+            if (!loadable(key0 + e)) v[e] = zero;
+          vreg[i] = v;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const int idx = tid + THREADS * i, cb = idx / 4, kg = idx % 4;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          treg[i][j] = zeros;
+          if (idx < (DV / 8) * 4 && loadable(kbase + 8 * kg + j))
+            treg[i][j] = *(const bf16x8*)(key_row(8 * kg + j) + 8 * cb);
+        }
+      }
+      if constexpr (RCH > 0) {
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+          const int idx = tid + THREADS * i, kl = idx / RCH, c8 = DV / 8 + idx % RCH;
+          rreg[i] = zeros;
+          if (idx < 32 * RCH && loadable(kbase + kl)) rreg[i] = *(const bf16x8*)(key_row(kl) + 8 * c8);
+        }
       }
     }
-    if (!VK) {
-      for (int idx = tid; idx < DV * 4; idx += THREADS) {
-        const int d = idx / 4, k8 = idx % 4, key0 = kbase + 8 * k8;
-        bf16x8 v = zeros;
-        if (key0 <= kmax && (key0 + 7 >= kmin || key0 < keep)) {
-          const int pg = table[key0 / page];
-          v = *(const bf16x8*)(a.vc + (((size_t)pg * nkv + kvh) * DV + d) * page + key0 % page);
+  };
+  auto store = [&]() {
+    if constexpr (!VK) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {                // a slot of the page that holds no visible key may hold anything
-            const int key = key0 + e;
-            if (!(key <= kmax && (key >= kmin || key < keep))) v[e] = zero;
+      for (int i = 0; i < NKC; ++i) {
+        const int idx = tid + THREADS * i, kl = idx / KCH, c8 = idx % KCH;
+        if (idx < 32 * KCH) *(bf16x8*)(ks + kl * KROW + 8 * c8) = kreg[i];
+      }
+#pragma unroll
+      for (int i = 0; i < NVC; ++i) {
+        const int idx = tid + THREADS * i, d = idx / 4, k8 = idx % 4;
+        if (idx < DV * 4) *(bf16x8*)(vt + d * VROW + 8 * k8) = vreg[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const int idx = tid + THREADS * i, cb = idx / 4, kg = idx % 4;
+        if (idx < (DV / 8) * 4) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) *(bf16x8*)(ks + (8 * kg + j) * KROW + 8 * cb) = treg[i][j];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {                // channel 8 cb + e of the tile's 8 keys
+            bf16x8 t;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) t[j] = treg[i][j][e];
+            *(bf16x8*)(vt + (8 * cb + e) * VROW + 8 * kg) = t;
           }
         }
-        *(bf16x8*)(vt + d * VROW + 8 * k8) = v;
+      }
+      if constexpr (RCH > 0) {
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+          const int idx = tid + THREADS * i, kl = idx / RCH, c8 = DV / 8 + idx % RCH;
+          if (idx < 32 * RCH) *(bf16x8*)(ks + kl * KROW + 8 * c8) = rreg[i];
+        }
       }
     }
+  };
+
+  if (i0 < i1) fetch(block_base(i0));
+  for (int i = i0; i < i1; ++i) {
+    const int kbase = block_base(i);
+    __syncthreads();                                   // the last block's readers are done
+    store();
     __syncthreads();
+    if (i + 1 < i1) fetch(block_base(i + 1));
+    if (!wave_live) continue;                          // (a wavefront without columns only helps staging)
 
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
     const __bf16* kp = ks + (8 * (n / 4) + n % 4) * KROW + 8 * gq;
@@ -153,26 +244,37 @@ __global__ __launch_bounds__(64 * NW) void window_attention_mfma_kernel(const Wi
       s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf[kk], s0, 0, 0, 0);
       s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf[kk], s1, 0, 0, 0);
     }
+    // score of key kbase + 8 gq + j: raw * scale - slope * (pos_c - key), in units of log 2
+    const float bias0 = -slope2 * (float)(pos_c - kbase - 8 * gq);
     float s[8], top = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int key = kbase + 8 * gq + j;
-      const bool sees = key <= pos_c && (key >= lo_c || key < a.keep_first);
-      const float raw = j < 4 ? s0[j] : s1[j - 4];
-      s[j] = sees ? raw * scale2 - slope2 * (float)(pos_c - key) : -INFINITY;
-      top = fmaxf(top, s[j]);
+    for (int j = 0; j < 8; ++j)
+      s[j] = fmaf(j < 4 ? s0[j] : s1[j - 4], scale2, fmaf(slope2, (float)j, bias0));
+    const bool whole = kbase + 31 <= pos_lo && (kbase >= lo_hi || kbase + 31 < a.keep_first);
+    if (!whole) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = kbase + 8 * gq + j;
+        if (!(key <= pos_c && (key >= lo_c || key < a.keep_first))) s[j] = -INFINITY;
+      }
     }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) top = fmaxf(top, s[j]);
     const float mn = fmaxf(m, column_max4(top));
-    // a column that has seen no key yet keeps m = -inf: nothing to rescale, nothing to add
-    const float alpha = mn == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - mn);
     float p[8], psum = 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      p[j] = s[j] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(s[j] - mn);
+    for (int j = 0; j < 8; ++j) {                      // exp2(-inf) = 0; mn = -inf only while no key was seen
+      p[j] = mn == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(s[j] - mn);
       psum += p[j];
     }
-    l = l * alpha + column_sum4(psum);
-    m = mn;
+    if (__any(mn > m)) {                               // the maximum of some column moved: rescale
+      const float alpha = mn == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - mn);
+      l *= alpha;
+#pragma unroll
+      for (int dd = 0; dd < DD; ++dd) o[dd] *= alpha;
+      m = mn;
+    }
+    l += column_sum4(psum);
     bf16x8 p1, p2, p3;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -184,7 +286,7 @@ __global__ __launch_bounds__(64 * NW) void window_attention_mfma_kernel(const Wi
 #pragma unroll
     for (int dd = 0; dd < DD; ++dd) {
       const bf16x8 vf = *(const bf16x8*)(vt + (16 * dd + n) * VROW + 8 * gq);
-      f32x4 acc = o[dd] * alpha;
+      f32x4 acc = o[dd];
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p3, acc, 0, 0, 0);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p2, acc, 0, 0, 0);
       o[dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p1, acc, 0, 0, 0);
@@ -223,15 +325,14 @@ __global__ __launch_bounds__(64 * NW) void window_attention_mfma_kernel(const Wi
   }
 }
 
-template <int NW>
 static const char* launch_mfma(const WindowAttention& a, dim3 grid, hipStream_t stream) {
   const size_t bytes = sizeof(__bf16) * ((size_t)32 * KROW + (size_t)DV * VROW);
   if (bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)window_attention_mfma_kernel<NW>,
+    hipError_t e = hipFuncSetAttribute((const void*)window_attention_mfma_kernel,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) return hipGetErrorString(e);
   }
-  window_attention_mfma_kernel<NW><<<grid, 64 * NW, bytes, stream>>>(a);
+  window_attention_mfma_kernel<<<grid, THREADS, bytes, stream>>>(a);
   return sl_launch_status();
 }
 
@@ -265,11 +366,10 @@ extern "C" const char* sl_window_attention_mfma(
                           cu_q, positions, nh, nkv, Dk, Dv, page, scale, window, keep_first, slopes, sinks,
                           (const act_t*)gate, gate_stride, (act_t*)out, nsplit, part_o, part_ml};
   const long long cols = (long long)max_q_len * (nh / nkv);
-  const int nw = cols <= 16 ? 1 : 4;
-  const long long tiles = (cols + 16 * nw - 1) / (16 * nw);
+  const long long tiles = (cols + COLS - 1) / COLS;
   SL_CHECK(tiles * nsplit <= 1 << 30, "window attention: too many column tiles");
   const dim3 grid((unsigned)(tiles * nsplit), nkv, num_seqs);
-  const char* e = nw == 1 ? launch_mfma<1>(a, grid, stream) : launch_mfma<4>(a, grid, stream);
+  const char* e = launch_mfma(a, grid, stream);
   if (e || nsplit == 1) return e;
   window_attention_combine_kernel<<<dim3(num_tokens, nh), 64, 0, stream>>>(
       part_o, part_ml, nsplit, nh, Dv, sinks, (const act_t*)gate, gate_stride, (act_t*)out);
