@@ -6,8 +6,12 @@
 // is taken to the latent's space (A[h] = Wuk[h]^T) and the attention's output
 // back from it (A[h] = Wuv[h]).
 //
-// A workgroup owns 64 tokens x 64 outputs of one head; K goes through LDS in
-// chunks of 16, every thread keeps 4 x 4 sums.
+// The general kernel: a workgroup owns 64 tokens x 64 outputs of one head; K goes
+// through LDS in chunks of 16, every thread keeps 4 x 4 sums.  bfloat16 with K in
+// steps of 32, N in steps of 16 and 16-byte aligned heads runs on the matrix cores:
+// a wavefront owns 16 tokens x 64 outputs and reads its operands straight from
+// memory, eight values a lane (rows of A are the first operand of mfma 16x16x32,
+// rows of x the second), so a step of a few single tokens reads every matrix once.
 #include "common.h"
 
 constexpr int HG_TILE = 64;
@@ -62,6 +66,52 @@ __global__ __launch_bounds__(256) void head_products_kernel(
   }
 }
 
+#if !defined(SL_F32)
+typedef __bf16 hg_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 hg_bf16x4 __attribute__((ext_vector_type(4)));
+typedef float hg_f32x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(64) void head_products_mfma_kernel(
+    const __bf16* __restrict__ x, long long x_row, int x_head, const __bf16* __restrict__ A,
+    __bf16* __restrict__ y, long long y_row, int y_head, int T, int N, int K) {
+  const int lane = threadIdx.x, i = lane & 15, gq = lane >> 4;
+  const int h = blockIdx.z, n0 = blockIdx.x * 64, t0 = blockIdx.y * 16;
+  const int t = t0 + i < T ? t0 + i : T - 1;           // rows past the last: computed like the last, never stored
+  const __bf16* xp = x + (size_t)t * x_row + (size_t)h * x_head + 8 * gq;
+  const __bf16* ap[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int n = n0 + 16 * u + i < N ? n0 + 16 * u + i : N - 1;
+    ap[u] = A + ((size_t)h * N + n) * K + 8 * gq;
+  }
+  hg_f32x4 acc[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) acc[u] = hg_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k = 0; k < K; k += 32) {
+    const hg_bf16x8 b = *(const hg_bf16x8*)(xp + k);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (n0 + 16 * u < N) {
+        const hg_bf16x8 a = *(const hg_bf16x8*)(ap[u] + k);
+        acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[u], 0, 0, 0);
+      }
+    }
+  }
+  if (t0 + i >= T) return;
+  // this lane holds outputs n0 + 16 u + 4 gq .. + 3 of token t0 + i
+  __bf16* yp = y + (size_t)(t0 + i) * y_row + (size_t)h * y_head + n0 + 4 * gq;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    if (n0 + 16 * u < N) {
+      hg_bf16x4 r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = (__bf16)acc[u][e];
+      *(hg_bf16x4*)(yp + 16 * u) = r;
+    }
+  }
+}
+#endif
+
 extern "C" const char* sl_head_products(const void* x, long long x_row, int x_head, const void* A,
                                         void* y, long long y_row, int y_head, int T, int heads, int N,
                                         int K, hipStream_t stream) {
@@ -71,6 +121,16 @@ extern "C" const char* sl_head_products(const void* x, long long x_row, int x_he
   SL_CHECK(x_row >= (long long)(heads - 1) * x_head + K && y_row >= (long long)(heads - 1) * y_head + N,
            "head_products: rows are shorter than their heads");
   if (T == 0) return nullptr;
+#if !defined(SL_F32)
+  if (K % 32 == 0 && N % 16 == 0 && (uintptr_t)x % 16 == 0 && x_row % 8 == 0 && x_head % 8 == 0 &&
+      (uintptr_t)A % 16 == 0 && (uintptr_t)y % 8 == 0 && y_row % 4 == 0 && y_head % 4 == 0 &&
+      (T + 15) / 16 <= 65535) {
+    const dim3 mgrid((N + 63) / 64, (T + 15) / 16, heads);
+    head_products_mfma_kernel<<<mgrid, 64, 0, stream>>>((const __bf16*)x, x_row, x_head, (const __bf16*)A,
+                                                        (__bf16*)y, y_row, y_head, T, N, K);
+    return sl_launch_status();
+  }
+#endif
   const dim3 grid((N + HG_TILE - 1) / HG_TILE, (T + HG_TILE - 1) / HG_TILE, heads);
   SL_CHECK(grid.y <= 65535, "head_products: too many rows");
   head_products_kernel<<<grid, 256, 0, stream>>>((const act_t*)x, x_row, x_head, (const act_t*)A,

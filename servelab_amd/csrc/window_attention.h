@@ -36,25 +36,33 @@ __global__ __launch_bounds__(64) void window_attention_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int nsplit, int nh, int Dv,
     const float* __restrict__ sinks, const act_t* __restrict__ gate, int gate_stride,
     act_t* __restrict__ out) {
+  __shared__ float ws[64];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const size_t base = ((size_t)t * nh + h) * nsplit;
-  float top = sinks != nullptr ? sinks[h] : -INFINITY;
-  for (int j = 0; j < nsplit; ++j) top = fmaxf(top, part_ml[(base + j) * 2]);
-  float denom = sinks != nullptr ? expf(sinks[h] - top) : 0.f;
-  for (int j = 0; j < nsplit; ++j) {
-    const float mj = part_ml[(base + j) * 2];
-    if (mj != -INFINITY) denom += expf(mj - top) * part_ml[(base + j) * 2 + 1];
+  // lane j holds share j (at most 64 shares)
+  float mj = -INFINITY, lj = 0.f;
+  if (lane < nsplit) {
+    mj = part_ml[(base + lane) * 2];
+    lj = part_ml[(base + lane) * 2 + 1];
   }
+  const float sink = sinks != nullptr ? sinks[h] : -INFINITY;
+  const float top = fmaxf(wave_max(mj), sink);
+  const float wj = mj == -INFINITY ? 0.f : expf(mj - top);
+  const float denom = wave_sum(wj * lj) + (sinks != nullptr ? expf(sink - top) : 0.f);
+  ws[lane] = wj;
+  __syncthreads();
   float f = 1.f / denom;
   if (gate != nullptr) f *= sigmoidf_(to_f(gate[(size_t)t * gate_stride + h]));
   act_t* o = out + ((size_t)t * nh + h) * Dv;
   for (int d = lane; d < Dv; d += 64) {
     float s = 0.f;
-    for (int j = 0; j < nsplit; ++j) {
-      const float mj = part_ml[(base + j) * 2];
-      if (mj != -INFINITY) s += expf(mj - top) * part_o[(base + j) * Dv + d];
+    for (int j = 0; j < nsplit; j += 8) {              // eight shares asked for together; added in their order
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = j + u < nsplit ? part_o[(base + j + u) * Dv + d] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += (j + u < nsplit ? ws[j + u] : 0.f) * v[u];
     }
     o[d] = from_f<act_t>(s * f);
   }
 }
-

@@ -17,7 +17,6 @@ class WindowOps:
     # (the float kernel, the matrix-core kernel)
     WINDOW_SHARE_KEYS = 256
     WINDOW_MAX_SHARES = 16
-    WINDOW_MFMA_SHARE_KEYS = 128
     WINDOW_MFMA_MAX_SHARES = 32
     WINDOW_MFMA_LDS_BYTES = 160 * 1024
 
@@ -208,8 +207,11 @@ class WindowOps:
         nsplit = 1
         if batch.max_q_len == 1:
             span = batch.max_ctx_len if not window else min(batch.max_ctx_len, window + int(keep_first))
-            nsplit = max(1, min(self.WINDOW_MFMA_MAX_SHARES, span // self.WINDOW_MFMA_SHARE_KEYS) if mfma
-                         else min(self.WINDOW_MAX_SHARES, span // self.WINDOW_SHARE_KEYS))
+            if mfma:
+                # a workgroup for every CU, a block of 32 keys a share at least
+                nsplit = max(1, min(self.WINDOW_MFMA_MAX_SHARES, span // 32, self._num_cus // max(1, S * nkv)))
+            else:
+                nsplit = max(1, min(self.WINDOW_MAX_SHARES, span // self.WINDOW_SHARE_KEYS))
         part_o = part_ml = None
         if nsplit > 1:
             part_o = self._new((T, nh, nsplit, Dv), torch.float32)

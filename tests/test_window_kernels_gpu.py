@@ -57,21 +57,25 @@ def test_add_layernorm(ops, T, H):
         close(out2, plain.layer_norm_gain(want_sum, gain.double(), 1e-5)[rows.long()], dt)
 
 
-@pytest.mark.parametrize("T,heads,N,K,pad", [(1, 3, 40, 16, 8), (7, 2, 5, 33, 0), (130, 4, 70, 24, 3), (64, 1, 64, 64, 0)])
-def test_head_products(ops, T, heads, N, K, pad):
+@pytest.mark.parametrize("T,heads,N,K,pad,col", [
+    (1, 3, 40, 16, 8, 5), (7, 2, 5, 33, 0, 5), (130, 4, 70, 24, 3, 5), (64, 1, 64, 64, 0, 5),
+    # aligned heads with K in steps of 32 and N in steps of 16: the matrix cores in bfloat16
+    (3, 5, 48, 32, 8, 8), (130, 2, 80, 96, 0, 0), (17, 3, 16, 64, 16, 16)])
+def test_head_products(ops, T, heads, N, K, pad, col):
     g = torch.Generator().manual_seed(T + N)
     dt = ops.act_dtype
-    x = torch.randn(T, 5 + heads * (K + pad), generator=g).to(dt)
+    x = torch.randn(T, col + heads * (K + pad), generator=g).to(dt)
     A = (torch.randn(heads, N, K, generator=g) / K ** 0.5).to(dt)
-    want = torch.einsum("thk,hnk->thn", x[:, 5:].view(T, heads, K + pad)[..., :K].double(), A.double())
-    y = ops.head_products(dev(x), 5, heads, K + pad, dev(A))
+    want = torch.einsum("thk,hnk->thn", x[:, col:].view(T, heads, K + pad)[..., :K].double(), A.double())
+    y = ops.head_products(dev(x), col, heads, K + pad, dev(A))
     close(y.view(T, heads, N), want, dt)
     # into columns of a wider buffer, which stays as it was elsewhere
-    wide = torch.full((T, 2 + heads * (N + 3)), 7.0).to(dt)
-    out = ops.head_products(dev(x), 5, heads, K + pad, dev(A), y=dev(wide), y_col=2, y_head=N + 3)
-    got = out[:, 2:].view(T, heads, N + 3)
+    gap = 3 if col == 5 else 4
+    wide = torch.full((T, 4 + heads * (N + gap)), 7.0).to(dt)
+    out = ops.head_products(dev(x), col, heads, K + pad, dev(A), y=dev(wide), y_col=4, y_head=N + gap)
+    got = out[:, 4:].view(T, heads, N + gap)
     close(got[..., :N], want, dt)
-    assert (got[..., N:] == 7).all() and (out[:, :2] == 7).all()
+    assert (got[..., N:] == 7).all() and (out[:, :4] == 7).all()
 
 
 def paged(seq_lens, page, nkv, Dk, Dv, dtype, gen, num_pages=None):
