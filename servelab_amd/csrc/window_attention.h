@@ -31,7 +31,7 @@ __device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-
 
 // Merges the shares of a (token, head): out = sum_j w_j o_j / (sum_j w_j l_j + sink's term),
 // w_j = exp(m_j - top); a share without keys has m = -inf and drops out.  One
-// wavefront per (token, head); shares are added in their order.
+// wavefront per (token, head, 64 channels); shares are added in their order.
 __global__ __launch_bounds__(64) void window_attention_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int nsplit, int nh, int Dv,
     const float* __restrict__ sinks, const act_t* __restrict__ gate, int gate_stride,
@@ -54,7 +54,8 @@ __global__ __launch_bounds__(64) void window_attention_combine_kernel(
   float f = 1.f / denom;
   if (gate != nullptr) f *= sigmoidf_(to_f(gate[(size_t)t * gate_stride + h]));
   act_t* o = out + ((size_t)t * nh + h) * Dv;
-  for (int d = lane; d < Dv; d += 64) {
+  const int d = blockIdx.z * 64 + lane;
+  if (d < Dv) {
     float s = 0.f;
     for (int j = 0; j < nsplit; j += 8) {              // eight shares asked for together; added in their order
       float v[8];

@@ -246,7 +246,7 @@ extern "C" const char* sl_window_attention(
     e = launch_window_attention<16>(a, grid, need(16), stream);
   }
   if (e || nsplit == 1) return e;
-  window_attention_combine_kernel<<<dim3(num_tokens, nh), 64, 0, stream>>>(
+  window_attention_combine_kernel<<<dim3(num_tokens, nh, (Dv + 63) / 64), 64, 0, stream>>>(
       part_o, part_ml, nsplit, nh, Dv, sinks, (const act_t*)gate, gate_stride, (act_t*)out);
   return sl_launch_status();
 }
