@@ -71,46 +71,59 @@ typedef __bf16 hg_bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 hg_bf16x4 __attribute__((ext_vector_type(4)));
 typedef float hg_f32x4 __attribute__((ext_vector_type(4)));
 
-// NU tiles of 16 outputs a wavefront: 4 for many tokens (a row of x serves 64 outputs), 1 for a
-// few single tokens (more wavefronts, each with a short chain of loads).
-template <int NU>
+// NT tiles of 16 tokens by NU tiles of 16 outputs a wavefront: 4 x 4 for many tokens (eight loads
+// feed sixteen matrix instructions), 1 x 1 for a few single tokens (more wavefronts, each with a
+// short chain of loads).
+template <int NT, int NU>
 __global__ __launch_bounds__(64) void head_products_mfma_kernel(
     const __bf16* __restrict__ x, long long x_row, int x_head, const __bf16* __restrict__ A,
     __bf16* __restrict__ y, long long y_row, int y_head, int T, int N, int K) {
   const int lane = threadIdx.x, i = lane & 15, gq = lane >> 4;
-  const int h = blockIdx.z, n0 = blockIdx.x * 16 * NU, t0 = blockIdx.y * 16;
-  const int t = t0 + i < T ? t0 + i : T - 1;           // rows past the last: computed like the last, never stored
-  const __bf16* xp = x + (size_t)t * x_row + (size_t)h * x_head + 8 * gq;
+  const int h = blockIdx.z, n0 = blockIdx.x * 16 * NU, t0 = blockIdx.y * 16 * NT;
+  const __bf16* xp[NT];
+#pragma unroll
+  for (int v = 0; v < NT; ++v) {                       // rows past the last: computed like the last, never stored
+    const int t = t0 + 16 * v + i < T ? t0 + 16 * v + i : T - 1;
+    xp[v] = x + (size_t)t * x_row + (size_t)h * x_head + 8 * gq;
+  }
   const __bf16* ap[NU];
 #pragma unroll
   for (int u = 0; u < NU; ++u) {
     const int n = n0 + 16 * u + i < N ? n0 + 16 * u + i : N - 1;
     ap[u] = A + ((size_t)h * N + n) * K + 8 * gq;
   }
-  hg_f32x4 acc[NU];
+  hg_f32x4 acc[NT][NU];
 #pragma unroll
-  for (int u = 0; u < NU; ++u) acc[u] = hg_f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
+  for (int v = 0; v < NT; ++v)
+#pragma unroll
+    for (int u = 0; u < NU; ++u) acc[v][u] = hg_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
   for (int k = 0; k < K; k += 32) {
-    const hg_bf16x8 b = *(const hg_bf16x8*)(xp + k);
+    hg_bf16x8 b[NT], a[NU];
+#pragma unroll
+    for (int v = 0; v < NT; ++v) b[v] = *(const hg_bf16x8*)(xp[v] + k);
+#pragma unroll
+    for (int u = 0; u < NU; ++u) a[u] = *(const hg_bf16x8*)(ap[u] + k);
+#pragma unroll
+    for (int v = 0; v < NT; ++v)
+#pragma unroll
+      for (int u = 0; u < NU; ++u)
+        acc[v][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[v], acc[v][u], 0, 0, 0);
+  }
+  // this lane holds outputs n0 + 16 u + 4 gq .. + 3 of tokens t0 + 16 v + i
+#pragma unroll
+  for (int v = 0; v < NT; ++v) {
+    const int t = t0 + 16 * v + i;
+    if (t >= T) continue;
+    __bf16* yp = y + (size_t)t * y_row + (size_t)h * y_head + n0 + 4 * gq;
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
       if (n0 + 16 * u < N) {
-        const hg_bf16x8 a = *(const hg_bf16x8*)(ap[u] + k);
-        acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[u], 0, 0, 0);
+        hg_bf16x4 r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = (__bf16)acc[v][u][e];
+        *(hg_bf16x4*)(yp + 16 * u) = r;
       }
-    }
-  }
-  if (t0 + i >= T) return;
-  // this lane holds outputs n0 + 16 u + 4 gq .. + 3 of token t0 + i
-  __bf16* yp = y + (size_t)(t0 + i) * y_row + (size_t)h * y_head + n0 + 4 * gq;
-#pragma unroll
-  for (int u = 0; u < NU; ++u) {
-    if (n0 + 16 * u < N) {
-      hg_bf16x4 r;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) r[e] = (__bf16)acc[u][e];
-      *(hg_bf16x4*)(yp + 16 * u) = r;
     }
   }
 }
@@ -128,12 +141,15 @@ extern "C" const char* sl_head_products(const void* x, long long x_row, int x_he
 #if !defined(SL_F32)
   if (K % 32 == 0 && N % 16 == 0 && (uintptr_t)x % 16 == 0 && x_row % 8 == 0 && x_head % 8 == 0 &&
       (uintptr_t)A % 16 == 0 && (uintptr_t)y % 8 == 0 && y_row % 4 == 0 && y_head % 4 == 0 &&
-      (T + 15) / 16 <= 65535) {
+      (T + 15) / 16 <= 65535) {   // (rows of A past N are clamped, their results never stored)
     if (T <= 16)
-      head_products_mfma_kernel<1><<<dim3(N / 16, 1, heads), 64, 0, stream>>>(
+      head_products_mfma_kernel<1, 1><<<dim3(N / 16, 1, heads), 64, 0, stream>>>(
+          (const __bf16*)x, x_row, x_head, (const __bf16*)A, (__bf16*)y, y_row, y_head, T, N, K);
+    else if (T <= 256)
+      head_products_mfma_kernel<1, 4><<<dim3((N + 63) / 64, (T + 15) / 16, heads), 64, 0, stream>>>(
           (const __bf16*)x, x_row, x_head, (const __bf16*)A, (__bf16*)y, y_row, y_head, T, N, K);
     else
-      head_products_mfma_kernel<4><<<dim3((N + 63) / 64, (T + 15) / 16, heads), 64, 0, stream>>>(
+      head_products_mfma_kernel<4, 4><<<dim3((N + 63) / 64, (T + 63) / 64, heads), 64, 0, stream>>>(
           (const __bf16*)x, x_row, x_head, (const __bf16*)A, (__bf16*)y, y_row, y_head, T, N, K);
     return sl_launch_status();
   }

@@ -202,11 +202,97 @@ __global__ void add_layernorm_kernel(float* __restrict__ resid, const act_t* __r
     o[i] = from_f<act_t>(((again ? value(i) : x[i]) - mean) * inv * w[i]);
 }
 
+// The same for rows of up to 4 * 8 * blockDim values that are a multiple of 4 wide: every value
+// is read once with 16-byte loads and stays in registers for the mean, the squared deviations
+// and the output.
+template <int ITERS>
+__global__ void add_layernorm_vec_kernel(float* __restrict__ resid, const act_t* __restrict__ d1,
+                                         const act_t* __restrict__ d2, const int* __restrict__ rows,
+                                         const float* __restrict__ w, act_t* __restrict__ out, int H,
+                                         float eps) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t src = rows != nullptr ? (size_t)rows[r] : (size_t)r;
+  float* x = resid + src * H;
+  const act_t* a = d1 != nullptr ? d1 + src * H : nullptr;
+  const act_t* b = d2 != nullptr ? d2 + src * H : nullptr;
+  const int H4 = H / 4;
+  f4 v[ITERS];
+  float sum = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int i = threadIdx.x + it * blockDim.x;
+    if (i < H4) {
+      v[it] = ((const f4*)x)[i];
+      if (a != nullptr || b != nullptr) {
+        float d[4] = {0.f, 0.f, 0.f, 0.f};
+        if (a != nullptr) {
+          const a4 av = ((const a4*)a)[i];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) d[j] = to_f(av.v[j]);
+        }
+        if (b != nullptr) {
+          const a4 bv = ((const a4*)b)[i];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) d[j] += to_f(bv.v[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[it].v[j] += d[j];
+        if (rows == nullptr) ((f4*)x)[i] = v[it];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sum += v[it].v[j];
+    }
+  }
+  const float mean = block_sum(sum, scratch) / (float)H;
+  float sq = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int i = threadIdx.x + it * blockDim.x;
+    if (i < H4) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[it].v[j] -= mean;
+        sq += v[it].v[j] * v[it].v[j];
+      }
+    }
+  }
+  const float inv = 1.f / sqrtf(block_sum(sq, scratch) / (float)H + eps);
+  act_t* o = out + (size_t)r * H;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int i = threadIdx.x + it * blockDim.x;
+    if (i < H4) {
+      const f4 wv = ((const f4*)w)[i];
+      a4 ov;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ov.v[j] = from_f<act_t>(v[it].v[j] * inv * wv.v[j]);
+      ((a4*)o)[i] = ov;
+    }
+  }
+}
+
 extern "C" const char* sl_add_layernorm(float* resid, const void* d1, const void* d2, const int* rows,
                                         const float* w, void* out, int R, int H, float eps,
                                         hipStream_t stream) {
   SL_CHECK(R >= 0 && H > 0, "add_layernorm: sizes must be positive");
   if (R == 0) return nullptr;
+  const bool aligned = ((uintptr_t)resid % 16) == 0 && ((uintptr_t)out % sizeof(a4)) == 0 &&
+                       ((uintptr_t)d1 % sizeof(a4)) == 0 && ((uintptr_t)d2 % sizeof(a4)) == 0 &&
+                       ((uintptr_t)w % 16) == 0;
+  if (H % 4 == 0 && H <= 4 * 8 * 512 && aligned) {
+    const int H4 = H / 4;
+    const int nthreads = H4 <= 64 ? 64 : (H4 <= 128 ? 128 : (H4 <= 256 ? 256 : 512));
+    const int iters = (H4 + nthreads - 1) / nthreads;
+    const act_t* a = (const act_t*)d1;
+    const act_t* b = (const act_t*)d2;
+    act_t* o = (act_t*)out;
+    if (iters == 1) add_layernorm_vec_kernel<1><<<R, nthreads, 0, stream>>>(resid, a, b, rows, w, o, H, eps);
+    else if (iters == 2) add_layernorm_vec_kernel<2><<<R, nthreads, 0, stream>>>(resid, a, b, rows, w, o, H, eps);
+    else if (iters <= 4) add_layernorm_vec_kernel<4><<<R, nthreads, 0, stream>>>(resid, a, b, rows, w, o, H, eps);
+    else add_layernorm_vec_kernel<8><<<R, nthreads, 0, stream>>>(resid, a, b, rows, w, o, H, eps);
+    return sl_launch_status();
+  }
   const int threads = H >= 2048 ? 512 : 256;
   add_layernorm_kernel<<<R, threads, 0, stream>>>(resid, (const act_t*)d1, (const act_t*)d2, rows, w,
                                                   (act_t*)out, H, eps);
