@@ -139,10 +139,17 @@ __global__ __launch_bounds__(THREADS) void window_attention_mfma_kernel(const Wi
 
   // A block travels pages -> registers -> LDS; the registers are filled for block i + 1 while block i
   // is computed from LDS.
+  // The pages of a block (of its keys 0..15 and 16..31) are asked for one block earlier still, so
+  // that a block costs one trip to memory and not two in a row; by a vector load (an even lane
+  // asks for the first, an odd lane for the second) so that the wait for it is not the wait for LDS.
+  const int page_shift = __builtin_ctz(page);
+  auto ask_pages = [&](int kbase) {
+    const int key = kbase + ((lane & 1) << 4);
+    return table[(key <= kmax ? key : kbase) >> page_shift];
+  };
   bf16x8 kreg[NKC], vreg[NVC], treg[NT][8], rreg[NR];
-  auto fetch = [&](int kbase) {
-    const int pgA = table[kbase / page];
-    const int pgB = kbase + 16 <= kmax ? table[(kbase + 16) / page] : pgA;
+  auto fetch = [&](int kbase, int asked) {
+    const int pgA = __builtin_amdgcn_readlane(asked, 0), pgB = __builtin_amdgcn_readlane(asked, 1);
     auto key_row = [&](int kl) {                       // start of the cache row of key kbase + kl
       const int pg = kl < 16 ? pgA : pgB;
       return a.kc + (((size_t)pg * nkv + kvh) * page + ((kbase + kl) & (page - 1))) * DK;
@@ -226,13 +233,20 @@ __global__ __launch_bounds__(THREADS) void window_attention_mfma_kernel(const Wi
     }
   };
 
-  if (i0 < i1) fetch(block_base(i0));
+  int asked = 0;
+  if (i0 < i1) {
+    fetch(block_base(i0), ask_pages(block_base(i0)));
+    if (i0 + 1 < i1) asked = ask_pages(block_base(i0 + 1));
+  }
   for (int i = i0; i < i1; ++i) {
     const int kbase = block_base(i);
     __syncthreads();                                   // the last block's readers are done
     store();
     __syncthreads();
-    if (i + 1 < i1) fetch(block_base(i + 1));
+    if (i + 1 < i1) {
+      fetch(block_base(i + 1), asked);
+      if (i + 2 < i1) asked = ask_pages(block_base(i + 2));
+    }
     if (!wave_live) continue;                          // (a wavefront without columns only helps staging)
 
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
