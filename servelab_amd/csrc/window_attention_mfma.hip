@@ -6,9 +6,9 @@
 // the matrix instruction (every product is exact in float); scale, distance bias, mask, the
 // running maximum and sum and the exponentials are float vector code.  A weight p is not rounded
 // to bfloat16 for the second product: it is cut into three bfloat16 terms p = p1 + p2 + p3 (each
-// the rounding of what the terms before left over), which carry the 24 bits of a float's
-// significand, and the weighted sum of the values is three matrix instructions, one per term,
-// on float accumulators.
+// the upper 16 bits of what the terms before left over, 8 bits of significand a term), which
+// together are the float exactly, and the weighted sum of the values is three matrix
+// instructions, one per term, on float accumulators.
 //
 // Work layout.  A column is a (token, query head) pair of one sequence and one kv head; a
 // wavefront owns 16 columns, a workgroup of four wavefronts 64 consecutive ones, and walks the
@@ -41,6 +41,7 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int DK = SL_DK, DV = SL_DV;
 constexpr bool VK = SL_VK != 0;
@@ -168,9 +169,11 @@ __global__ __launch_bounds__(THREADS) void window_attention_mfma_kernel(const Wi
         if (idx < DV * 4 && key0 <= kmax && (key0 + 7 >= kmin || key0 < keep)) {
           const int pg = k8 < 2 ? pgA : pgB;
           bf16x8 v = *(const bf16x8*)(a.vc + (((size_t)pg * nkv + kvh) * DV + d) * page + (key0 & (page - 1)));
+          if (!((key0 + 7 <= kmax && key0 >= kmin) || key0 + 7 < keep)) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)                  // a slot of the page that holds no visible key may hold anything
-            if (!loadable(key0 + e)) v[e] = zero;
+            for (int e = 0; e < 8; ++e)                // a slot of the page that holds no visible key may hold anything
+              if (!loadable(key0 + e)) v[e] = zero;
+          }
           vreg[i] = v;
         }
       }
@@ -289,14 +292,26 @@ __global__ __launch_bounds__(THREADS) void window_attention_mfma_kernel(const Wi
       m = mn;
     }
     l += column_sum4(psum);
-    bf16x8 p1, p2, p3;
+    // p = p1 + p2 + p3 exactly: each term is the upper 16 bits (a bfloat16) of what the terms before left
+    // over, 8 bits of significand a term; two terms of neighbouring keys share a register
+    u32x4 w1, w2, w3;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      p1[j] = (__bf16)p[j];
-      const float r1 = p[j] - (float)p1[j];
-      p2[j] = (__bf16)r1;
-      p3[j] = (__bf16)(r1 - (float)p2[j]);
+    for (int j = 0; j < 8; j += 2) {
+      unsigned t1[2], t2[2], t3[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const float x = p[j + e];
+        t1[e] = __float_as_uint(x) & 0xffff0000u;
+        const float r1 = x - __uint_as_float(t1[e]);
+        t2[e] = __float_as_uint(r1) & 0xffff0000u;
+        t3[e] = __float_as_uint(r1 - __uint_as_float(t2[e]));
+      }
+      w1[j / 2] = __builtin_amdgcn_perm(t1[1], t1[0], 0x07060302u);
+      w2[j / 2] = __builtin_amdgcn_perm(t2[1], t2[0], 0x07060302u);
+      w3[j / 2] = __builtin_amdgcn_perm(t3[1], t3[0], 0x07060302u);
     }
+    const bf16x8 p1 = __builtin_bit_cast(bf16x8, w1), p2 = __builtin_bit_cast(bf16x8, w2),
+                 p3 = __builtin_bit_cast(bf16x8, w3);
 #pragma unroll
     for (int dd = 0; dd < DD; ++dd) {
       const bf16x8 vf = *(const bf16x8*)(vt + (16 * dd + n) * VROW + 8 * gq);
