@@ -216,6 +216,10 @@ class ProductOps:
         w = self.rows_of(weight)
         if M <= self.ROWS_KERNEL_MAX_M and K % 8 == 0:
             return self.linear_rows(x, w, bias, out_f32)
+        if K % 8:
+            # rows that are no multiple of 16 bytes: the plain tiled kernel for any number of rows (no
+            # library call, so that a captured decode step stays clear of it as well)
+            return self.linear_tiled(x, w, bias, out_f32)
         if out_f32:
             if M <= 4 * self.ROWS_KERNEL_MAX_M and K % 8 == 0:
                 return self.linear_rows(x, w, bias, out_f32)

@@ -59,7 +59,14 @@ MODEL_D = config(64, 211, 1e-5, [
     latent(3, 16, 16, 24, 48, 13, 0),
     attention(4, 2, 32, 16, 40, 0, True, 64),
 ])
-MODELS = {"A": MODEL_A, "B": MODEL_B, "C": MODEL_C, "D": MODEL_D}
+# sizes that are multiples of nothing convenient: a width of 100, a vocabulary of 97, heads of 12 and 20 channels,
+# a latent of 22 with 6 rotated channels of which 4 turn
+MODEL_E = config(100, 97, 1e-5, [
+    attention(5, 5, 12, 20, 7, 2, True, 52),
+    latent(2, 10, 6, 14, 22, 9, 36, base=77.0, dims=4),
+    attention(10, 5, 12, 20, 64, 1, True, 0),
+])
+MODELS = {"A": MODEL_A, "B": MODEL_B, "C": MODEL_C, "D": MODEL_D, "E": MODEL_E}
 
 
 def tensor_shapes(cfg):
