@@ -106,7 +106,13 @@ __global__ __launch_bounds__(THREADS) void window_attention_mfma_kernel(const Wi
   const int nblk = nA + nB;
   const int i0 = (int)((long long)nblk * share / a.nsplit);
   const int i1 = (int)((long long)nblk * (share + 1) / a.nsplit);
-  auto block_base = [&](int i) { return (i < nA ? i : firstB + (i - nA)) * 32; };
+  // The blocks are walked from the nearest keys to the farthest (the kept first tokens last): a distance
+  // bias makes nearer keys score higher, so the running maximum settles in the first block or two and
+  // the sums are rarely rescaled; without a bias the order does not matter.
+  auto block_base = [&](int i) {
+    const int b = nblk - 1 - i;
+    return (b < nA ? b : firstB + (b - nA)) * 32;
+  };
   auto loadable = [&](int key) { return key <= kmax && (key >= kmin || key < keep); };
 
   // this wavefront's columns, and this lane's (a column past the last is computed like the last, never stored)
