@@ -1,2 +1,2 @@
 """Importing this package registers the architectures it holds."""
-from . import qwen2, topelorn  # noqa: F401
+from . import qwen2, topelorn, vekanex  # noqa: F401

@@ -1,9 +1,11 @@
 from .base import (Block, Embedding, FeedForward, Mixer, Norm, PagedKVSpec, ParamSpec, Part,
                    PositionEncoding, RotaryLayout, RotaryTables, Runtime, StateSpec, prefixed)
-from .norm import RMSNorm
+from .norm import LayerNorm, PostRMSNorm, RMSNorm
 from .position import NoPosition, RotaryPosition
-from .attention import PagedAttention
+from .attention import PagedAttention, ProjectionNormAttention
 from .feedforward import GatedMLP
-from .block import PreNormBlock
+from .routed import RoutedExperts
+from .recurrent import GatedDeltaRule, GatedLinearAttention, MatrixLSTM, SideBySide
+from .block import ParallelBlock, PostNormBlock, PreNormBlock
 from .embedding import OutputHead, TokenEmbedding
 from .model import DecoderModel, LayerCall, ModelSpec, build_model_spec

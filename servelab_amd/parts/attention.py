@@ -92,3 +92,78 @@ class PagedAttention(Mixer):
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v,
             cache.page_size, group.block_tables, batch, self.score_scale, self.window,
             self.w_o, None, defer=True)
+
+
+class ProjectionNormAttention(Mixer):
+    """Grouped-query softmax attention whose q and k are RMS-normed over the whole projection
+    (all heads of a token at once, a gain of that size) before the rotation, with biases on q,
+    k, v and the output, keys of ``key_dim`` and values of ``value_dim`` channels, a score
+    scale given from outside and float32 softmax weights.  The position encoding turns the
+    leading channels of a head in halves.  Causal; ``window`` None keeps every key."""
+    graph_safe = True
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "out": "o", "q_bias": "q.b", "k_bias": "k.b",
+             "v_bias": "v.b", "out_bias": "o.b", "q_norm": "q.norm", "k_norm": "k.norm"}
+
+    def __init__(self, hidden_size, num_heads, num_kv_heads, key_dim, value_dim, scale, position,
+                 norm_eps, bias=True, window=None, names=None):
+        if num_heads % num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        self.hidden_size = int(hidden_size)
+        self.num_heads, self.num_kv_heads = int(num_heads), int(num_kv_heads)
+        self.key_dim, self.value_dim = int(key_dim), int(value_dim)
+        self.scale, self.norm_eps = float(scale), float(norm_eps)
+        self.position = position
+        self.bias = bool(bias)
+        self.window = None if not window else int(window)
+        self.names = dict(self.NAMES, **(names or {}))
+
+    def param_specs(self):
+        n, h = self.names, self.hidden_size
+        H, G, D, Dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        specs = {n["q"]: ParamSpec((H * D, h)), n["k"]: ParamSpec((G * D, h)), n["v"]: ParamSpec((G * Dv, h)),
+                 n["q_norm"]: ParamSpec((H * D,), init="gain"), n["k_norm"]: ParamSpec((G * D,), init="gain"),
+                 n["out"]: ParamSpec((h, H * Dv))}
+        if self.bias:
+            specs.update({n["q_bias"]: ParamSpec((H * D,)), n["k_bias"]: ParamSpec((G * D,)),
+                          n["v_bias"]: ParamSpec((G * Dv,)), n["out_bias"]: ParamSpec((h,))})
+        return specs
+
+    def cache_spec(self):
+        return PagedKVSpec(self.num_kv_heads, self.key_dim, self.window, value_dim=self.value_dim)
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        n = self.names
+        self.position.load(tensors, rt)
+        layout = self.position.layout()
+        if layout is not None and (layout.pairing != "half" or layout.rot_dim > self.key_dim):
+            raise ValueError("the rotation must turn leading channels of a head in halves")
+        self.rot = 0 if layout is None else int(layout.rot_dim)
+        w = torch.cat([tensors(n["q"]), tensors(n["k"]), tensors(n["v"])], 0)
+        extra = -w.shape[0] % 8
+        if extra:
+            w = torch.cat([w, w.new_zeros(extra, w.shape[1])], 0)
+        self.w_in = rt.linear_weight(w)
+        self.b_in = self.b_o = None
+        if self.bias:
+            b = torch.cat([tensors(n["q_bias"]).float(), tensors(n["k_bias"]).float(),
+                           tensors(n["v_bias"]).float(), torch.zeros(extra)], 0)
+            self.b_in = rt.vector(b)
+            self.b_o = rt.vector(tensors(n["out_bias"]))
+        self.q_gain = rt.vector(tensors(n["q_norm"]))
+        self.k_gain = rt.vector(tensors(n["k_norm"]))
+        self.w_o = rt.linear_weight(tensors(n["out"]), delta=True)
+
+    def forward(self, x, batch, cache, shared):
+        ops = self.rt.ops
+        H, G, D, Dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        group = batch.groups[cache.group]
+        buf = ops.linear(x, self.w_in, self.b_in, out_f32=True)
+        tables = self.position.tables(batch, shared) if self.rot else None
+        q = ops.projnorm_rope_store(buf, H, G, D, Dv, self.q_gain, self.k_gain, self.norm_eps, self.rot,
+                                    tables, group.slots if cache.write else None, cache.k, cache.v,
+                                    cache.page_size)
+        attn = ops.window_attention(q, 0, H, G, D, Dv, cache.k, cache.v, cache.page_size,
+                                    group.block_tables, batch, self.scale, self.window)
+        return ops.linear(attn, self.w_o, self.b_o)

@@ -87,3 +87,67 @@ class ParallelBlock(Block):
         if self.feedforward is None:
             return a
         return (a, self.feedforward.forward(x))
+
+
+class PostNormBlock(Block):
+    """h += m * Norm1(Mixer(h)); h += m * Norm2(FeedForward(h)): the norms sit on the sublayers'
+    outputs (``PostRMSNorm`` parts, which hold m), and the sublayers read the stream itself, as
+    rows in the activation dtype that the norm's kernel writes along with its add.  The block
+    leaves no pending delta.  ``feedforward`` may be None.  A mixer made of several mixers
+    declares its cache needs as a list (``cache_specs``) and gets the list of bindings.
+
+    The rows of the stream travel from block to block in the step's ``shared`` dict; a block of
+    another kind that changes the stream has to drop the entry ``"stream rows"``."""
+
+    def __init__(self, norm1, mixer, norm2, feedforward, names=("norm1.", "mix.", "norm2.", "mlp.")):
+        self.norm1, self.mixer, self.norm2, self.feedforward = norm1, mixer, norm2, feedforward
+        self.names = tuple(names)
+
+    @property
+    def graph_safe(self):
+        return all(part.graph_safe for _, part in self._children())
+
+    def _children(self):
+        parts = [(self.names[0], self.norm1), (self.names[1], self.mixer)]
+        if self.feedforward is not None:
+            parts += [(self.names[2], self.norm2), (self.names[3], self.feedforward)]
+        return parts
+
+    def cache_specs(self):
+        several = getattr(self.mixer, "cache_specs", None)
+        if several is not None:
+            return list(several())
+        spec = self.mixer.cache_spec()
+        return [] if spec is None else [spec]
+
+    def param_specs(self):
+        specs = {}
+        for prefix, part in self._children():
+            for name, spec in part.param_specs().items():
+                specs[prefix + name] = spec
+        return specs
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        for prefix, part in self._children():
+            part.load(prefixed(prefix, tensors), rt)
+
+    def forward(self, resid, delta, batch, caches, shared):
+        ops = self.rt.ops
+        x = shared.get("stream rows")
+        if delta is not None:                 # what a block of another kind left to be added
+            for d in (delta if isinstance(delta, (tuple, list)) else (delta,)):
+                if d is not None:
+                    ops.add_into(resid, ops.materialize(d))
+            x = None
+        if x is None:
+            x = self.norm1.forward_post(resid, None)
+        if hasattr(self.mixer, "cache_specs"):
+            y = self.mixer.forward(x, batch, caches, shared)
+        else:
+            y = self.mixer.forward(x, batch, caches[0] if caches else None, shared)
+        x = self.norm1.forward_post(resid, ops.materialize(y))
+        if self.feedforward is not None:
+            x = self.norm2.forward_post(resid, ops.materialize(self.feedforward.forward(x)))
+        shared["stream rows"] = x
+        return None

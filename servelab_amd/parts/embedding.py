@@ -31,24 +31,31 @@ class OutputHead(Part):
     graph_safe = True
     takes_scaled_rows = True
 
-    """``tied_to`` is the embedding part whose table the head shares, or None."""
+    """``tied_to`` is the embedding part whose table the head shares, or None.
+    ``softcap`` c: the logits become c * tanh(logits / c), in float32."""
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to=None):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to=None, name: str = "weight",
+                 softcap=None):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.tied_to = tied_to
+        self.name = name
+        self.softcap = float(softcap) if softcap else None
 
     def param_specs(self):
         if self.tied_to is not None:
             return {}
-        return {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+        return {self.name: ParamSpec((self.vocab_size, self.hidden_size))}
 
     def load(self, tensors, rt):
         self.rt = rt
         if self.tied_to is not None:
             self.weight = rt.linear_weight(self.tied_to.weight, shared=True)
         else:
-            self.weight = rt.linear_weight(tensors("weight"))
+            self.weight = rt.linear_weight(tensors(self.name))
 
     def forward(self, rows):
         """normed rows [R, H] -> float32 logits [R, V]."""
-        return self.rt.ops.linear(rows, self.weight, None, out_f32=True)
+        logits = self.rt.ops.linear(rows, self.weight, None, out_f32=True)
+        if self.softcap is not None:
+            logits = self.rt.ops.softcap(logits, self.softcap)
+        return logits

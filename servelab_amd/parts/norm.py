@@ -54,3 +54,18 @@ class LayerNorm(Norm):
 
     def forward_rows(self, resid, delta, rows, fuse=False):
         return self.rt.ops.add_layernorm(resid, delta, self.weight, self.eps, rows=rows)
+
+
+class PostRMSNorm(RMSNorm):
+    """An RMS norm on a sublayer's output instead of its input: the stream takes
+    ``mult`` times the normed output, and the sublayers read the stream itself.
+    ``forward_post(resid, y)`` adds mult * norm(y) into the float32 stream in
+    place and returns the stream's rows in the activation dtype, which is what
+    the next sublayer reads (``y`` None: only those rows)."""
+
+    def __init__(self, size: int, eps: float, mult: float = 1.0, name: str = "weight"):
+        super().__init__(size, eps, name)
+        self.mult = float(mult)
+
+    def forward_post(self, resid, y):
+        return self.rt.ops.add_postnorm(resid, y, self.weight, self.eps, self.mult)

@@ -161,6 +161,227 @@ class EmulatedOps:
             out[a:b] = o.reshape(b - a, nh * D).to(self.act_dtype)
         return out
 
+    # ------------------------------------------- deltas, norms on outputs
+    def materialize(self, value):
+        return value
+
+    def add_into(self, resid, delta):
+        resid += _f(delta)
+
+    def add_postnorm(self, resid, y, weight, eps, mult):
+        """resid += mult * y / sqrt(mean(y^2) + eps) * weight; returns the stream's rows in the
+        activation dtype (y None: only those)."""
+        if y is not None:
+            y = _f(y)
+            resid += mult * (y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps) * weight)
+        return resid.to(self.act_dtype)
+
+    def scaled_sum(self, a, sa, b, sb):
+        return (sa * _f(a) + sb * _f(b)).to(self.act_dtype)
+
+    def softcap(self, logits, cap):
+        return logits.copy_(cap * torch.tanh(logits / cap))
+
+    # --------------------------------------------- matrix memories in state slots
+    @staticmethod
+    def _sequences(batch):
+        """(first row, one past the last row, state slot, whether the sequence starts here)."""
+        cu, slots, pos = batch.cu_q.tolist(), batch.state_slots.tolist(), batch.positions.tolist()
+        return [(cu[s], cu[s + 1], slots[s], pos[cu[s]] == 0) for s in range(batch.num_seqs)]
+
+    def lowrank_expand(self, buf, col, w2, bias, mode, heads=1, divisor=1.0, rates=None):
+        """z = buf[:, col:col + rank] w2^T + bias, float32 [T, C]; "plain": z; "log_sigmoid":
+        logsigmoid(z) / divisor; "rate_softplus": -exp(rates[h]) softplus(z), h = c // (C / heads)."""
+        C, rank = w2.shape
+        z = buf[:, col:col + rank].float() @ w2.T
+        if bias is not None:
+            z = z + bias
+        if mode == "plain":
+            return z
+        if mode == "log_sigmoid":
+            return torch.nn.functional.logsigmoid(z) / divisor
+        if mode == "rate_softplus":
+            rate = torch.exp(rates).repeat_interleave(C // heads)
+            return -rate * torch.nn.functional.softplus(z)
+        raise ValueError(mode)
+
+    def short_conv(self, buf, col, taps, state, state_off, batch, write, unit_heads=0, unit_dim=0,
+                   unit_eps=1e-6, scaled_heads=0, scale=1.0):
+        """silu of a causal convolution over time per channel of buf[:, col:col + C] (taps [C, n],
+        the last tap is the token's own); the n - 1 inputs before a step's first token come from
+        state[slot, state_off:] laid out [n - 1, C] (oldest first; zeros at a sequence's start) and
+        the step's last n - 1 inputs go back there.  The first ``unit_heads`` heads of ``unit_dim``
+        channels are then divided by sqrt(sum x^2 + unit_eps); the first ``scaled_heads`` of them
+        also multiplied by ``scale``."""
+        C, n = taps.shape
+        x = buf[:, col:col + C].float()
+        out = torch.empty_like(x)
+        for a, b, slot, fresh in self._sequences(batch):
+            keep = state[slot, state_off:state_off + (n - 1) * C].view(n - 1, C)
+            past = torch.zeros(n - 1, C) if fresh else keep.clone()
+            full = torch.cat([past, x[a:b]], 0)
+            y = sum(full[j:j + b - a] * taps[:, j] for j in range(n))
+            out[a:b] = y * torch.sigmoid(y)
+            if write and n > 1:
+                keep.copy_(full[full.shape[0] - (n - 1):])
+        if unit_heads:
+            heads = out[:, :unit_heads * unit_dim].view(-1, unit_heads, unit_dim)
+            heads /= torch.sqrt(heads.pow(2).sum(-1, keepdim=True) + unit_eps)
+            heads[:, :scaled_heads] *= scale
+        return out
+
+    def decay_scan(self, src, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, beta_src, beta_col,
+                   state, batch, write):
+        """Per head S' = diag(exp(log_decay)) S + k v^T and o = S'^T (q_scale q); with
+        ``beta_src``: S' = diag(..) S, u = sigmoid(beta) (v - S'^T k), S' += k u^T.  q and k have G
+        heads (head h reads h // (H / G)).  The state slot holds S as [H, Dv, D] from 0 on."""
+        T = src.shape[0]
+        q = src[:, q_col:q_col + G * D].float().view(T, G, D) * q_scale
+        k = src[:, k_col:k_col + G * D].float().view(T, G, D)
+        v = src[:, v_col:v_col + H * Dv].float().view(T, H, Dv)
+        decay = torch.exp(log_decay.view(T, H, D))
+        out = torch.empty(T, H, Dv)
+        rep = H // G
+        for a, b, slot, fresh in self._sequences(batch):
+            kept = state[slot, :H * Dv * D].view(H, Dv, D)
+            S = torch.zeros(H, Dv, D) if fresh else kept.clone()
+            for t in range(a, b):
+                kt, qt = k[t].repeat_interleave(rep, 0), q[t].repeat_interleave(rep, 0)
+                S = S * decay[t][:, None, :]
+                if beta_src is None:
+                    u = v[t]
+                else:
+                    beta = torch.sigmoid(beta_src[t, beta_col:beta_col + H].float())
+                    u = beta[:, None] * (v[t] - torch.einsum("hvd,hd->hv", S, kt))
+                S = S + u[:, :, None] * kt[:, None, :]
+                out[t] = torch.einsum("hvd,hd->hv", S, qt)
+            if write:
+                kept.copy_(S)
+        return out.view(T, H * Dv)
+
+    def mlstm_scan(self, buf, q_col, k_col, v_col, i_col, f_col, H, D, Dv, cap, q_scale, state, batch,
+                   write):
+        """Matrix memory with exponential gates and a running maximum that starts at 0; the slot
+        holds S [H, Dv, D], then n [H, D], then m [H].  Returns S'^T q / (max(|n' . q|, e^-m') + 1e-6)."""
+        T = buf.shape[0]
+        q = buf[:, q_col:q_col + H * D].float().view(T, H, D) * q_scale
+        k = buf[:, k_col:k_col + H * D].float().view(T, H, D)
+        v = buf[:, v_col:v_col + H * Dv].float().view(T, H, Dv)
+        ig = cap * torch.tanh(buf[:, i_col:i_col + H].float() / cap)
+        fg = torch.nn.functional.logsigmoid(cap * torch.tanh(buf[:, f_col:f_col + H].float() / cap))
+        out = torch.empty(T, H, Dv)
+        nS, nn = H * Dv * D, H * D
+        for a, b, slot, fresh in self._sequences(batch):
+            row = state[slot]
+            if fresh:
+                S, n, m = torch.zeros(H, Dv, D), torch.zeros(H, D), torch.zeros(H)
+            else:
+                S, n, m = row[:nS].view(H, Dv, D).clone(), row[nS:nS + nn].view(H, D).clone(), row[nS + nn:nS + nn + H].clone()
+            for t in range(a, b):
+                new = torch.maximum(fg[t] + m, ig[t])
+                keep, add = torch.exp(fg[t] + m - new), torch.exp(ig[t] - new)
+                S = keep[:, None, None] * S + add[:, None, None] * v[t][:, :, None] * k[t][:, None, :]
+                n = keep[:, None] * n + add[:, None] * k[t]
+                m = new
+                den = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+                out[t] = torch.einsum("hvd,hd->hv", S, q[t]) / den[:, None]
+            if write:
+                row[:nS].copy_(S.reshape(-1))
+                row[nS:nS + nn].copy_(n.reshape(-1))
+                row[nS + nn:nS + nn + H].copy_(m)
+        return out.view(T, H * Dv)
+
+    def head_norm_gate(self, o, H, Dv, weight, per_head, eps, gate, gate_col, activation):
+        """Each head of o [T, H Dv] (float32) divided by its root mean square, times ``weight``
+        ([H Dv] when ``per_head``, else [Dv] for every head), times sigmoid or silu of
+        gate[:, gate_col:gate_col + H Dv]."""
+        T = o.shape[0]
+        x = o.view(T, H, Dv)
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        x = x * (weight.view(H, Dv) if per_head else weight)
+        g = gate[:, gate_col:gate_col + H * Dv].float().view(T, H, Dv)
+        g = torch.sigmoid(g) if activation == "sigmoid" else g * torch.sigmoid(g)
+        return (x * g).reshape(T, H * Dv).to(self.act_dtype)
+
+    # -------------------------------------- attention with a norm over the projection
+    def projnorm_rope_store(self, buf, H, G, D, Dv, q_gain, k_gain, eps, rot, tables, slots, k_cache,
+                            v_cache, page_size):
+        """buf (float32) holds q [H D], k [G D], v [G Dv] side by side.  q and k are RMS-normed over
+        all their heads at once, their heads' first ``rot`` channels rotated in halves; k and v go
+        to the pages, q is returned [T, H D]."""
+        T = buf.shape[0]
+
+        def normed(x, gain):
+            return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * gain
+
+        def turned(x):
+            if not rot:
+                return x
+            half = rot // 2
+            c, s = tables.cos[:, None, :], tables.sin[:, None, :]
+            a, b = x[..., :half], x[..., half:rot]
+            return torch.cat([a * c - b * s, b * c + a * s, x[..., rot:]], -1)
+        q = turned(normed(buf[:, :H * D].float(), q_gain).view(T, H, D))
+        k = turned(normed(buf[:, H * D:(H + G) * D].float(), k_gain).view(T, G, D))
+        v = buf[:, (H + G) * D:(H + G) * D + G * Dv].float().view(T, G, Dv)
+        if slots is not None:
+            page, off = (slots // page_size).long(), (slots % page_size).long()
+            k_cache[page, :, off, :] = k.to(k_cache.dtype)
+            v_cache[page, :, :, off] = v.to(v_cache.dtype)
+        return q.reshape(T, H * D).to(self.act_dtype)
+
+    def window_attention(self, q, q_col, nh, nkv, Dk, Dv, k_cache, v_cache, page_size, block_tables,
+                         batch, scale, window, keep_first=0, slopes=None, sinks=None, gate=None,
+                         gate_col=0):
+        if slopes is not None or sinks is not None or gate is not None or v_cache is None:
+            raise NotImplementedError("the emulated window attention has no bias, sink, gate or latent")
+        T = q.shape[0]
+        g = nh // nkv
+        out = torch.empty(T, nh * Dv, dtype=self.act_dtype)
+        cu, ctxs = batch.cu_q.tolist(), batch.ctx_len.tolist()
+        for s in range(batch.num_seqs):
+            a, b = cu[s], cu[s + 1]
+            qs = _f(q[a:b, q_col:q_col + nh * Dk]).view(b - a, nh, Dk)
+            q_pos = batch.positions[a:b].long()
+            k_pos = torch.arange(0, ctxs[s])
+            vis = k_pos[None, :] <= q_pos[:, None]
+            if window:
+                vis &= (k_pos[None, :] > q_pos[:, None] - window) | (k_pos[None, :] < keep_first)
+            seen = vis.any(0)
+            k_pos, vis = k_pos[seen], vis[:, seen]             # released pages are never read
+            pages = block_tables[s].long()[k_pos // page_size]
+            offs = k_pos % page_size
+            k = _f(k_cache[pages, :, offs, :]).repeat_interleave(g, dim=1)
+            v = _f(v_cache[pages, :, :, offs]).repeat_interleave(g, dim=1)
+            scores = torch.einsum("qhd,rhd->hqr", qs, k) * scale
+            scores = scores.masked_fill(~vis[None], float("-inf"))
+            o = torch.einsum("hqr,rhd->qhd", torch.softmax(scores, -1), v)
+            out[a:b] = o.reshape(b - a, nh * Dv).to(self.act_dtype)
+        return out
+
+    # ------------------------------------------------------- routed experts
+    def route_tokens(self, logits, experts, top):
+        """The ``top`` largest of a row's first ``experts`` logits (float32; ties to the lower
+        index) and the softmax over them: (chosen [T, top] int32, shares [T, top] float32)."""
+        z = logits[:, :experts].float()
+        best = torch.topk(z, top, dim=-1, sorted=True)
+        return best.indices.to(torch.int32), torch.softmax(best.values, -1)
+
+    def routed_experts(self, x, routing, w_gate_up, w_down, base=None):
+        """sum over a token's choices of share * down_e(silu(gate_e x) * up_e x) (+ base);
+        w_gate_up [E, 2 ff, width] holds an expert's gate rows before its up rows."""
+        chosen, shares = routing
+        T = x.shape[0]
+        ff = w_gate_up.shape[1] // 2
+        xf = _f(x)
+        out = torch.zeros(T, w_down.shape[1]) if base is None else _f(base).clone()
+        for t in range(T):
+            for e, s in zip(chosen[t].tolist(), shares[t].tolist()):
+                gu = _f(w_gate_up[e]) @ xf[t]
+                mid = (gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]).to(self.act_dtype).float()
+                out[t] += s * (_f(w_down[e]) @ mid)
+        return out.to(self.act_dtype)
+
     # ------------------------------------------------------------- sampling
     def argmax(self, logits):
         return torch.argmax(logits, dim=-1).to(torch.int32)
