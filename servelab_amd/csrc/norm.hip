@@ -311,3 +311,69 @@ extern "C" const char* sl_add_into(float* resid, const void* delta, long long n,
   add_into_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(resid, (const act_t*)delta, (size_t)n);
   return sl_launch_status();
 }
+
+// RMS norm on a sublayer's output: resid (float, in place) += mult * y * rsqrt(mean(y^2) + eps) * w,
+// and the stream's new rows in the activation type for the sublayer that reads them next.  y == nullptr:
+// only those rows.  One block per row; sums and the stream in float.
+__global__ void add_postnorm_kernel(float* __restrict__ resid, const act_t* __restrict__ y,
+                                    const float* __restrict__ w, act_t* __restrict__ out, int H, float eps,
+                                    float mult) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  float* x = resid + r * H;
+  act_t* o = out + r * H;
+  if (y == nullptr) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = from_f<act_t>(x[i]);
+    return;
+  }
+  const act_t* yr = y + r * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float v = to_f(yr[i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.f / sqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float v = x[i] + mult * (to_f(yr[i]) * inv * w[i]);
+    x[i] = v;
+    o[i] = from_f<act_t>(v);
+  }
+}
+
+extern "C" const char* sl_add_postnorm(float* resid, const void* y, const float* w, void* out, int T, int H,
+                                       float eps, float mult, hipStream_t stream) {
+  SL_CHECK(T >= 0 && H > 0, "add_postnorm: sizes must be positive");
+  if (T == 0) return nullptr;
+  add_postnorm_kernel<<<T, H >= 2048 ? 512 : 256, 0, stream>>>(resid, (const act_t*)y, w, (act_t*)out, H, eps, mult);
+  return sl_launch_status();
+}
+
+// out = sa * a + sb * b, float sums: the outputs of two mixers that ran side by side.
+__global__ void scaled_sum_kernel(const act_t* __restrict__ a, float sa, const act_t* __restrict__ b, float sb,
+                                  act_t* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_f<act_t>(sa * to_f(a[i]) + sb * to_f(b[i]));
+}
+
+extern "C" const char* sl_scaled_sum(const void* a, float sa, const void* b, float sb, void* out, long long n,
+                                     hipStream_t stream) {
+  SL_CHECK(n >= 0, "scaled_sum: the count must not be negative");
+  if (n == 0) return nullptr;
+  scaled_sum_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((const act_t*)a, sa, (const act_t*)b, sb,
+                                                                    (act_t*)out, (size_t)n);
+  return sl_launch_status();
+}
+
+// x = cap * tanh(x / cap) in place on float values (logits).
+__global__ void softcap_kernel(float* __restrict__ x, float cap, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = cap * tanhf(x[i] / cap);
+}
+
+extern "C" const char* sl_softcap(float* x, float cap, long long n, hipStream_t stream) {
+  SL_CHECK(n >= 0 && cap > 0.f, "softcap: the count must not be negative, the cap positive");
+  if (n == 0) return nullptr;
+  softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, cap, (size_t)n);
+  return sl_launch_status();
+}

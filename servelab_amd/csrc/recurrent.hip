@@ -1,0 +1,441 @@
+// Mixers whose memory is a matrix per head in a state slot: what runs between their input
+// projection (float sums [T, width]) and their output projection.
+//
+//   lowrank_expand   z = t W2^T + b from the few columns a low-rank projection left, as a log
+//                    decay (logsigmoid(z) / tau, or -exp(rate_h) softplus(z)) or plain
+//   short_conv       silu of a causal convolution over time per channel, the last taps - 1
+//                    inputs kept in the state slot; heads made unit vectors
+//   matrix_scan      the recurrences: decay per key channel (S' = diag(a) S + k v^T), the same
+//                    with the delta rule's correction (u = beta (v - S'^T k)), and the matrix
+//                    LSTM (scalar gates with a running maximum, a normaliser n)
+//   head_norm_gate   a head's read-out divided by its root mean square, gain, output gate
+//   projnorm_rope_store  softmax attention's q and k normed over the whole projection, rotated,
+//                    k and v written to their pages
+//
+// Everything here is float: gates, decays and their logarithms, unit norms, the state, the
+// read-out.  The activation type appears only where rows leave for a matrix product or a page.
+//
+// State layout: S as [head][value channel][key channel] (a column of the matrix, which one
+// lane group owns, is contiguous), then what the mixer keeps besides.
+#include "common.h"
+
+__device__ __forceinline__ float softplusf_(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+__device__ __forceinline__ float logsigmoidf_(float x) { return -softplusf_(-x); }
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
+
+// ------------------------------------------------------------------ low-rank expansion
+// out[t][c] = f(sum_r buf[t][col + r] W2[c][r] + bias[c]);  mode 0: z, 1: logsigmoid(z) / divisor,
+// 2: -exp(rates[c / per_head]) * softplus(z)
+__global__ void lowrank_expand_kernel(const float* __restrict__ buf, int stride, int col, int rank,
+                                      const float* __restrict__ w2, const float* __restrict__ bias, int C,
+                                      int mode, float divisor, const float* __restrict__ rates, int per_head,
+                                      float* __restrict__ out) {
+  extern __shared__ float low[];
+  const size_t t = blockIdx.x;
+  for (int r = threadIdx.x; r < rank; r += blockDim.x) low[r] = buf[t * stride + col + r];
+  __syncthreads();
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const float* w = w2 + (size_t)c * rank;
+  float z = 0.f;
+  for (int r = 0; r < rank; ++r) z += low[r] * w[r];
+  if (bias != nullptr) z += bias[c];
+  if (mode == 1) z = logsigmoidf_(z) / divisor;
+  else if (mode == 2) z = -expf(rates[c / per_head]) * softplusf_(z);
+  out[t * C + c] = z;
+}
+
+extern "C" const char* sl_lowrank_expand(const float* buf, int stride, int col, int rank, const float* w2,
+                                         const float* bias, int T, int C, int mode, float divisor,
+                                         const float* rates, int heads, float* out, hipStream_t stream) {
+  SL_CHECK(T >= 0 && C > 0 && rank > 0 && rank <= 8192, "lowrank_expand: sizes must be positive, rank <= 8192");
+  SL_CHECK(col >= 0 && col + rank <= stride, "lowrank_expand: the columns do not fit the rows");
+  SL_CHECK(mode >= 0 && mode <= 2 && heads > 0 && C % heads == 0, "lowrank_expand: unknown mode or heads");
+  SL_CHECK(mode != 2 || rates != nullptr, "lowrank_expand: rates are missing");
+  SL_CHECK(mode != 1 || divisor > 0.f, "lowrank_expand: the divisor must be positive");
+  if (T == 0) return nullptr;
+  lowrank_expand_kernel<<<dim3(T, (C + 255) / 256), 256, rank * sizeof(float), stream>>>(
+      buf, stride, col, rank, w2, bias, C, mode, divisor, rates, C / heads, out);
+  return sl_launch_status();
+}
+
+// ------------------------------------------------------------------ short convolution
+struct ShortConv {
+  const float* buf;          // inputs of token t at buf + t * stride + col
+  int stride, col, C, taps;
+  const float* w;            // [C][taps], the last tap is the token's own
+  float* state;              // slot s at state + s * state_stride + state_off: [taps - 1][C], oldest first
+  long long state_stride;
+  int state_off;
+  const int* cu_q;
+  const int* positions;
+  const int* tok_seq;
+  const int* slots;
+  int unit_heads, unit_dim, scaled_heads;
+  float unit_eps, scale;
+  float* out;                // [T][C]
+};
+
+// One wavefront per (token, head of the unit part | 256 other channels).
+__global__ __launch_bounds__(64) void short_conv_kernel(const ShortConv a) {
+  const int t = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+  int c0, n;
+  if (b < a.unit_heads) {
+    c0 = b * a.unit_dim;
+    n = a.unit_dim;
+  } else {
+    c0 = a.unit_heads * a.unit_dim + (b - a.unit_heads) * 256;
+    n = min(256, a.C - c0);
+  }
+  const int s = a.tok_seq[t];
+  const int first = a.cu_q[s];
+  const int i = t - first;                                  // place of the token in its step
+  const bool fresh = a.positions[first] == 0;               // the sequence starts in this step
+  const float* past = a.state + (size_t)a.slots[s] * a.state_stride + a.state_off;
+  const int back = a.taps - 1;
+  float ss = 0.f;
+  float y[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int c = c0 + lane + u * 64;
+    y[u] = 0.f;
+    if (lane + u * 64 < n) {
+      float acc = 0.f;
+      for (int j = 0; j < a.taps; ++j) {
+        const int idx = i - back + j;                       // place in the step of the tap's input
+        float x;
+        if (idx >= 0) x = a.buf[(size_t)(first + idx) * a.stride + a.col + c];
+        else x = fresh ? 0.f : past[(size_t)(back + idx) * a.C + c];
+        acc += a.w[(size_t)c * a.taps + j] * x;
+      }
+      y[u] = acc * sigmoidf_(acc);
+      ss += y[u] * y[u];
+    }
+  }
+  float f = 1.f;
+  if (b < a.unit_heads) {
+    ss = wave_sum(ss);
+    f = 1.f / sqrtf(ss + a.unit_eps);
+    if (b < a.scaled_heads) f *= a.scale;
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    if (lane + u * 64 < n) a.out[(size_t)t * a.C + c0 + lane + u * 64] = y[u] * f;
+}
+
+// The slot's new last inputs, after the kernel above has read the old ones: a thread per
+// (sequence, channel) walks the rows oldest first; row r takes what lies len rows later, which
+// is either a row it has not written yet or an input of this step.
+__global__ void short_conv_state_kernel(const ShortConv a, int S) {
+  const int s = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= a.C) return;
+  const int first = a.cu_q[s], len = a.cu_q[s + 1] - first;
+  const bool fresh = a.positions[first] == 0;
+  float* keep = a.state + (size_t)a.slots[s] * a.state_stride + a.state_off;
+  const int back = a.taps - 1;
+  for (int r = 0; r < back; ++r) {
+    const int idx = len - back + r;
+    float x;
+    if (idx >= 0) x = a.buf[(size_t)(first + idx) * a.stride + a.col + c];
+    else x = fresh ? 0.f : keep[(size_t)(back + idx) * a.C + c];
+    keep[(size_t)r * a.C + c] = x;
+  }
+}
+
+extern "C" const char* sl_short_conv(const float* buf, int stride, int col, int C, int taps, const float* w,
+                                     float* state, long long state_stride, int state_off, const int* cu_q,
+                                     const int* positions, const int* tok_seq, const int* slots, int S, int T,
+                                     int write, int unit_heads, int unit_dim, float unit_eps, int scaled_heads,
+                                     float scale, float* out, hipStream_t stream) {
+  SL_CHECK(T >= 0 && S >= 0 && C > 0 && taps >= 1 && taps <= 64, "short_conv: sizes must be positive, taps <= 64");
+  SL_CHECK(col >= 0 && col + C <= stride, "short_conv: the channels do not fit the rows");
+  SL_CHECK(unit_heads >= 0 && (unit_heads == 0 || (unit_dim >= 1 && unit_dim <= 256)) &&
+           (long long)unit_heads * unit_dim <= C && scaled_heads <= unit_heads,
+           "short_conv: unit heads of at most 256 channels within the channels");
+  SL_CHECK(state_off >= 0 && state_off + (long long)(taps - 1) * C <= state_stride,
+           "short_conv: the last inputs do not fit the state slot");
+  if (T == 0) return nullptr;
+  const ShortConv a{buf, stride, col, C, taps, w, state, state_stride, state_off, cu_q, positions, tok_seq,
+                    slots, unit_heads, unit_dim, scaled_heads, unit_eps, scale, out};
+  const int rest = C - unit_heads * unit_dim;
+  short_conv_kernel<<<dim3(T, unit_heads + (rest + 255) / 256), 64, 0, stream>>>(a);
+  if (write && taps > 1) short_conv_state_kernel<<<dim3(S, (C + 255) / 256), 256, 0, stream>>>(a, S);
+  return sl_launch_status();
+}
+
+// ------------------------------------------------------------------ the recurrences
+struct MatrixScan {
+  const float* src;          // q, k, v of token t at src + t * src_stride + {q,k,v}_col; q and k have G heads
+  int src_stride, q_col, k_col, v_col;
+  int H, G, D, Dv;
+  const float* log_decay;    // [T][H][D] (decay and delta modes)
+  float q_scale;
+  const float* gates;        // delta: beta before its sigmoid at gates + t * gate_stride + beta_col + h;
+  int gate_stride, i_col, f_col;   // matrix LSTM: the two gates before cap and squashing at i_col + h, f_col + h
+  float cap;
+  float* state;              // slot s at state + s * state_stride: S [H][Dv][D]; matrix LSTM: then n [H][D], m [H]
+  long long state_stride;
+  const int* cu_q;
+  const int* positions;
+  const int* slots;
+  int write;
+  float* out;                // [T][H][Dv]
+};
+
+enum { SCAN_DECAY = 0, SCAN_DELTA = 1, SCAN_LSTM = 2 };
+#define SCAN_ROWS 8          // key channels a lane owns: channels p, p + P, ..., p + 7 P
+
+// A block of 256 threads takes a (sequence, head, slice of value channels): P lanes share a
+// column of S (P a power of two with 8 P >= D), 256 / P columns a block.  The step's tokens go
+// through LDS a chunk at a time (q, k, decay of the head, v of the block's columns, gates); the
+// columns then walk the chunk token by token, a lane updating its 8 rows and the P lanes of a
+// column adding their parts of the read-out by butterfly.
+template <int MODE>
+__global__ __launch_bounds__(256) void matrix_scan_kernel(const MatrixScan a, int P, int CH) {
+  extern __shared__ float lds[];
+  const int s = blockIdx.x, h = blockIdx.y, slice = blockIdx.z, tid = threadIdx.x;
+  const int Dp = P * SCAN_ROWS, cols = 256 / P;
+  float* sq = lds;                       // [CH][Dp]
+  float* sk = sq + CH * Dp;              // [CH][Dp]
+  float* sa = sk + CH * Dp;              // [CH][Dp] decays (not for the matrix LSTM)
+  float* sv = MODE == SCAN_LSTM ? sa : sa + CH * Dp;     // [CH][cols]
+  float* sg = sv + CH * cols;            // [CH][2] gates
+  const int p = tid % P, cl = tid / P;
+  const int j = slice * cols + cl;
+  const bool live = j < a.Dv;
+  const int g = h / (a.H / a.G);
+  const int first = a.cu_q[s], last = a.cu_q[s + 1];
+  const bool fresh = a.positions[first] == 0;
+  float* slot = a.state + (size_t)a.slots[s] * a.state_stride;
+  float* col = slot + ((size_t)h * a.Dv + (live ? j : 0)) * a.D;
+  const size_t nS = (size_t)a.H * a.Dv * a.D;
+  float* nrow = slot + nS + (size_t)h * a.D;
+  float* mcell = slot + nS + (size_t)a.H * a.D + h;
+  float S[SCAN_ROWS], n[SCAN_ROWS];
+  float m = 0.f;
+#pragma unroll
+  for (int i = 0; i < SCAN_ROWS; ++i) {
+    const int r = i * P + p;
+    S[i] = (!fresh && live && r < a.D) ? col[r] : 0.f;
+    n[i] = (MODE == SCAN_LSTM && !fresh && r < a.D) ? nrow[r] : 0.f;
+  }
+  if (MODE == SCAN_LSTM && !fresh) m = *mcell;
+
+  for (int t0 = first; t0 < last; t0 += CH) {
+    const int nt = min(CH, last - t0);
+    __syncthreads();
+    for (int idx = tid; idx < nt * Dp; idx += 256) {
+      const int tt = idx / Dp, r = idx % Dp;
+      const size_t t = t0 + tt;
+      float q = 0.f, k = 0.f, d = 1.f;
+      if (r < a.D) {
+        q = a.src[t * a.src_stride + a.q_col + g * a.D + r] * a.q_scale;
+        k = a.src[t * a.src_stride + a.k_col + g * a.D + r];
+        if (MODE != SCAN_LSTM) d = expf(a.log_decay[(t * a.H + h) * a.D + r]);
+      }
+      sq[idx] = q;
+      sk[idx] = k;
+      if (MODE != SCAN_LSTM) sa[idx] = d;
+    }
+    for (int idx = tid; idx < nt * cols; idx += 256) {
+      const int tt = idx / cols, c = slice * cols + idx % cols;
+      sv[idx] = c < a.Dv ? a.src[(size_t)(t0 + tt) * a.src_stride + a.v_col + h * a.Dv + c] : 0.f;
+    }
+    if (MODE != SCAN_DECAY && tid < nt) {
+      const float* gr = a.gates + (size_t)(t0 + tid) * a.gate_stride;
+      if (MODE == SCAN_DELTA) {
+        sg[tid * 2] = sigmoidf_(gr[a.i_col + h]);
+      } else {
+        sg[tid * 2] = a.cap * tanhf(gr[a.i_col + h] / a.cap);
+        sg[tid * 2 + 1] = logsigmoidf_(a.cap * tanhf(gr[a.f_col + h] / a.cap));
+      }
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float* q = sq + tt * Dp;
+      const float* k = sk + tt * Dp;
+      const float* d = sa + tt * Dp;
+      const float v = sv[tt * cols + cl];
+      float o = 0.f, aux = 0.f;
+      if (MODE == SCAN_DECAY) {
+#pragma unroll
+        for (int i = 0; i < SCAN_ROWS; ++i) {
+          const int r = i * P + p;
+          S[i] = d[r] * S[i] + k[r] * v;
+          o += S[i] * q[r];
+        }
+      } else if (MODE == SCAN_DELTA) {
+#pragma unroll
+        for (int i = 0; i < SCAN_ROWS; ++i) {
+          const int r = i * P + p;
+          S[i] *= d[r];
+          aux += S[i] * k[r];
+        }
+        for (int w = 1; w < P; w <<= 1) aux += __shfl_xor(aux, w, SL_WAVE);
+        const float u = sg[tt * 2] * (v - aux);
+#pragma unroll
+        for (int i = 0; i < SCAN_ROWS; ++i) {
+          const int r = i * P + p;
+          S[i] += k[r] * u;
+          o += S[i] * q[r];
+        }
+      } else {
+        const float ig = sg[tt * 2], fg = sg[tt * 2 + 1];
+        const float top = fmaxf(fg + m, ig);
+        const float keep = expf(fg + m - top), add = expf(ig - top);
+        m = top;
+#pragma unroll
+        for (int i = 0; i < SCAN_ROWS; ++i) {
+          const int r = i * P + p;
+          const float ak = add * k[r];
+          S[i] = keep * S[i] + ak * v;
+          n[i] = keep * n[i] + ak;
+          o += S[i] * q[r];
+          aux += n[i] * q[r];
+        }
+      }
+      for (int w = 1; w < P; w <<= 1) o += __shfl_xor(o, w, SL_WAVE);
+      if (MODE == SCAN_LSTM) {
+        for (int w = 1; w < P; w <<= 1) aux += __shfl_xor(aux, w, SL_WAVE);
+        o = o / (fmaxf(fabsf(aux), expf(-m)) + 1e-6f);
+      }
+      if (p == 0 && live) a.out[((size_t)(t0 + tt) * a.H + h) * a.Dv + j] = o;
+    }
+  }
+  if (a.write) {
+#pragma unroll
+    for (int i = 0; i < SCAN_ROWS; ++i) {
+      const int r = i * P + p;
+      if (live && r < a.D) col[r] = S[i];
+      if (MODE == SCAN_LSTM && slice == 0 && cl == 0 && r < a.D) nrow[r] = n[i];
+    }
+    if (MODE == SCAN_LSTM && slice == 0 && tid == 0) *mcell = m;
+  }
+}
+
+extern "C" const char* sl_matrix_scan(int mode, const float* src, int src_stride, int q_col, int k_col, int v_col,
+                                      int H, int G, int D, int Dv, const float* log_decay, float q_scale,
+                                      const float* gates, int gate_stride, int i_col, int f_col, float cap,
+                                      float* state, long long state_stride, const int* cu_q, const int* positions,
+                                      const int* slots, int S, int T, int write, float* out, hipStream_t stream) {
+  SL_CHECK(mode >= 0 && mode <= 2, "matrix_scan: unknown mode");
+  SL_CHECK(S >= 0 && T >= 0 && H > 0 && G > 0 && H % G == 0 && Dv > 0, "matrix_scan: sizes must be positive");
+  SL_CHECK(D >= 1 && D <= 64 * SCAN_ROWS, "matrix_scan: at most 512 key channels a head");
+  SL_CHECK(q_col >= 0 && k_col >= 0 && v_col >= 0 && q_col + G * D <= src_stride && k_col + G * D <= src_stride &&
+           v_col + H * Dv <= src_stride, "matrix_scan: q, k or v do not fit the rows");
+  SL_CHECK(mode == SCAN_LSTM || log_decay != nullptr, "matrix_scan: decays are missing");
+  SL_CHECK(mode == SCAN_DECAY || (gates != nullptr && i_col >= 0 && i_col + H <= gate_stride),
+           "matrix_scan: gates are missing or do not fit their rows");
+  SL_CHECK(mode != SCAN_LSTM || (f_col >= 0 && f_col + H <= gate_stride && cap > 0.f),
+           "matrix_scan: the forget gates do not fit their rows");
+  const long long need = (long long)H * Dv * D + (mode == SCAN_LSTM ? (long long)H * D + H : 0);
+  SL_CHECK(need <= state_stride, "matrix_scan: the state does not fit its slot");
+  if (S == 0 || T == 0) return nullptr;
+  int P = 1;
+  while (P * SCAN_ROWS < D) P <<= 1;
+  const int cols = 256 / P, Dp = P * SCAN_ROWS;
+  const int CH = Dp <= 128 ? 16 : (Dp <= 256 ? 8 : 4);
+  const size_t lds = (size_t)CH * ((mode == SCAN_LSTM ? 2 : 3) * Dp + cols + 2) * sizeof(float);
+  const MatrixScan a{src, src_stride, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, gates, gate_stride,
+                     i_col, f_col, cap, state, state_stride, cu_q, positions, slots, write, out};
+  const dim3 grid(S, H, (Dv + cols - 1) / cols);
+  if (mode == SCAN_DECAY) matrix_scan_kernel<SCAN_DECAY><<<grid, 256, lds, stream>>>(a, P, CH);
+  else if (mode == SCAN_DELTA) matrix_scan_kernel<SCAN_DELTA><<<grid, 256, lds, stream>>>(a, P, CH);
+  else matrix_scan_kernel<SCAN_LSTM><<<grid, 256, lds, stream>>>(a, P, CH);
+  return sl_launch_status();
+}
+
+// ------------------------------------------------------------------ read-out: norm, gain, gate
+// One wavefront per (token, head): o / sqrt(mean(o^2) + eps) * w * act(gate); act 0: sigmoid, 1: silu.
+__global__ __launch_bounds__(64) void head_norm_gate_kernel(const float* __restrict__ o, int H, int Dv,
+                                                            const float* __restrict__ w, int per_head, float eps,
+                                                            const float* __restrict__ gate, int gate_stride,
+                                                            int gate_col, int act, act_t* __restrict__ out) {
+  const size_t t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const float* x = o + (t * H + h) * Dv;
+  float ss = 0.f;
+  for (int d = lane; d < Dv; d += 64) ss += x[d] * x[d];
+  const float inv = 1.f / sqrtf(wave_sum(ss) / (float)Dv + eps);
+  const float* gr = gate + t * gate_stride + gate_col + h * Dv;
+  const float* wr = w + (per_head ? h * Dv : 0);
+  for (int d = lane; d < Dv; d += 64) {
+    const float z = gr[d];
+    const float gv = act == 0 ? sigmoidf_(z) : z * sigmoidf_(z);
+    out[(t * H + h) * Dv + d] = from_f<act_t>(x[d] * inv * wr[d] * gv);
+  }
+}
+
+extern "C" const char* sl_head_norm_gate(const float* o, int T, int H, int Dv, const float* w, int per_head,
+                                         float eps, const float* gate, int gate_stride, int gate_col, int act,
+                                         void* out, hipStream_t stream) {
+  SL_CHECK(T >= 0 && H > 0 && Dv > 0, "head_norm_gate: sizes must be positive");
+  SL_CHECK(gate_col >= 0 && gate_col + H * Dv <= gate_stride, "head_norm_gate: the gates do not fit their rows");
+  SL_CHECK(act == 0 || act == 1, "head_norm_gate: the gate is sigmoid (0) or silu (1)");
+  if (T == 0) return nullptr;
+  head_norm_gate_kernel<<<dim3(T, H), 64, 0, stream>>>(o, H, Dv, w, per_head, eps, gate, gate_stride, gate_col,
+                                                       act, (act_t*)out);
+  return sl_launch_status();
+}
+
+// ------------------------------------------------------------------ softmax attention's q, k, v
+// buf row: q [H][D], k [G][D], v [G][Dv] (float).  q and k are divided by the root mean square of
+// all their heads together and multiplied by a gain of that size, then the first `rot` channels
+// of every head turn in halves (channel i with i + rot / 2, angle of cos/sin column i).  q leaves
+// in the activation type; k and v go to the token's place in the pages.  One block per token.
+__global__ void projnorm_rope_store_kernel(const float* __restrict__ buf, int stride, int H, int G, int D, int Dv,
+                                           const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+                                           int rot, const float* __restrict__ cosv, const float* __restrict__ sinv,
+                                           const int* __restrict__ slots, act_t* __restrict__ kc,
+                                           act_t* __restrict__ vc, int page, act_t* __restrict__ q_out) {
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  const float* row = buf + t * stride;
+  const int nq = H * D, nk = G * D, nv = G * Dv;
+  float sq = 0.f, sk = 0.f;
+  for (int e = threadIdx.x; e < nq; e += blockDim.x) sq += row[e] * row[e];
+  for (int e = threadIdx.x; e < nk; e += blockDim.x) sk += row[nq + e] * row[nq + e];
+  const float iq = 1.f / sqrtf(block_sum(sq, scratch) / (float)nq + eps);
+  const float ik = 1.f / sqrtf(block_sum(sk, scratch) / (float)nk + eps);
+  const int half = rot / 2;
+  const float* cs = cosv != nullptr ? cosv + t * half : nullptr;
+  const float* sn = sinv != nullptr ? sinv + t * half : nullptr;
+  const int slot = slots != nullptr ? slots[t] : 0;
+  const size_t pg = slot / page, off = slot % page;
+  for (int e = threadIdx.x; e < nq + nk; e += blockDim.x) {
+    const bool is_q = e < nq;
+    const int el = is_q ? e : e - nq;
+    const float* x = is_q ? row : row + nq;
+    const float* w = is_q ? qw : kw;
+    const float inv = is_q ? iq : ik;
+    const int d = el % D;
+    float v = x[el] * inv * w[el];
+    if (d < rot) {
+      const int i = d < half ? d : d - half;
+      const int partner = d < half ? el + half : el - half;
+      const float o = x[partner] * inv * w[partner];
+      v = d < half ? v * cs[i] - o * sn[i] : v * cs[i] + o * sn[i];
+    }
+    if (is_q) q_out[t * nq + el] = from_f<act_t>(v);
+    else if (slots != nullptr) kc[((pg * G + el / D) * page + off) * D + d] = from_f<act_t>(v);
+  }
+  if (slots != nullptr)
+    for (int e = threadIdx.x; e < nv; e += blockDim.x)
+      vc[((pg * G + e / Dv) * Dv + e % Dv) * page + off] = from_f<act_t>(row[nq + nk + e]);
+}
+
+extern "C" const char* sl_projnorm_rope_store(const float* buf, int stride, int T, int H, int G, int D, int Dv,
+                                              const float* qw, const float* kw, float eps, int rot,
+                                              const float* cosv, const float* sinv, const int* slots, void* kc,
+                                              void* vc, int page, void* q_out, hipStream_t stream) {
+  SL_CHECK(T >= 0 && H > 0 && G > 0 && D > 0 && Dv > 0 && page > 0, "projnorm_rope_store: sizes must be positive");
+  SL_CHECK((long long)(H + G) * D + (long long)G * Dv <= stride, "projnorm_rope_store: q, k and v do not fit the rows");
+  SL_CHECK(rot >= 0 && rot % 2 == 0 && rot <= D, "projnorm_rope_store: the rotated width must be even and within a head");
+  SL_CHECK(rot == 0 || (cosv != nullptr && sinv != nullptr), "projnorm_rope_store: cos and sin are missing");
+  SL_CHECK(slots == nullptr || (kc != nullptr && vc != nullptr), "projnorm_rope_store: pages are missing");
+  if (T == 0) return nullptr;
+  projnorm_rope_store_kernel<<<T, 256, 0, stream>>>(buf, stride, H, G, D, Dv, qw, kw, eps, rot, cosv, sinv, slots,
+                                                    (act_t*)kc, (act_t*)vc, page, (act_t*)q_out);
+  return sl_launch_status();
+}

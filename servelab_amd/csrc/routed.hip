@@ -1,0 +1,228 @@
+// Routed experts: every token goes through the `top` experts with the largest router logits,
+// weighted by the softmax over those logits only.
+//
+//   route       per token the chosen experts and their shares (float), one wavefront a token
+//   group       the step's (token, choice) pairs sorted by expert, on the device: where each
+//               expert's rows start, the list of row tiles (expert, first row, rows) that the
+//               grouped products walk, and each pair's place in the sorted order
+//   grouped     y[row] = W[expert of row] x[row]: one launch over all experts, a workgroup per
+//               (row tile, column tile); the gated form computes silu(gate) * up of an expert's
+//               stacked [gate; up] matrix
+//   combine     out[token] = base[token] + sum over its choices of share * y[place of the pair]
+//
+// No launch depends on the routing: the grids are sized for the worst case (pairs / tile rows
+// + experts tiles) and workgroups beyond the tiles in use leave at once, so a step is a fixed
+// list of launches that a captured graph can replay.
+#include "common.h"
+
+#define RT_ROWS 16           // rows of a tile of the grouped products
+
+// ------------------------------------------------------------------ route
+// One wavefront per token.  Largest first; among equal logits the lower index wins.
+__global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ logits, int stride, int E, int top,
+                                                   int* __restrict__ chosen, float* __restrict__ shares) {
+  const size_t t = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float* z = logits + t * stride;
+  unsigned long long taken = 0ull;             // bit u: element lane + 64 u is chosen already (E <= 4096)
+  float mine = 0.f;                            // lane k keeps the k-th largest logit
+  int mine_e = 0;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int u = 0, e = lane; e < E; ++u, e += 64) {
+      const float v = z[e];
+      if (!((taken >> u) & 1ull) && (v > best || (v == best && e < at))) {
+        best = v;
+        at = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, SL_WAVE);
+      const int oa = __shfl_xor(at, o, SL_WAVE);
+      if (ob > best || (ob == best && oa < at)) {
+        best = ob;
+        at = oa;
+      }
+    }
+    if (at % 64 == lane) taken |= 1ull << (at / 64);
+    if (lane == k) {
+      mine = best;
+      mine_e = at;
+    }
+  }
+  const float top1 = __shfl(mine, 0, SL_WAVE);
+  const float w = lane < top ? expf(mine - top1) : 0.f;
+  const float sum = wave_sum(w);
+  if (lane < top) {
+    chosen[t * top + lane] = mine_e;
+    shares[t * top + lane] = w / sum;
+  }
+}
+
+// ------------------------------------------------------------------ group
+// One workgroup sorts the n = tokens * top pairs by expert (counting sort in LDS).
+//   order[place] = pair (token * top + choice);  place_of[pair] = place
+//   tiles[i] = {expert, first row, rows} for i < tiles in use; rows 0 beyond
+__global__ __launch_bounds__(1024) void group_kernel(const int* __restrict__ chosen, int n, int E, int max_tiles,
+                                                     int* __restrict__ order, int* __restrict__ place_of,
+                                                     int* __restrict__ tiles) {
+  extern __shared__ int sh[];
+  int* count = sh;               // [E]
+  int* start = sh + E;           // [E] first row of the expert
+  int* tile0 = sh + 2 * E;       // [E] first tile of the expert
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += blockDim.x) count[e] = 0;
+  for (int i = tid; i < max_tiles; i += blockDim.x) {
+    tiles[3 * i] = 0;
+    tiles[3 * i + 1] = 0;
+    tiles[3 * i + 2] = 0;
+  }
+  __syncthreads();
+  for (int i = tid; i < n; i += blockDim.x) atomicAdd(&count[chosen[i]], 1);
+  __syncthreads();
+  if (tid == 0) {
+    int rows = 0, nt = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = rows;
+      tile0[e] = nt;
+      rows += count[e];
+      nt += (count[e] + RT_ROWS - 1) / RT_ROWS;
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += blockDim.x) {
+    const int c = count[e];
+    for (int i = 0; i * RT_ROWS < c; ++i) {
+      int* tl = tiles + 3 * (tile0[e] + i);
+      tl[0] = e;
+      tl[1] = start[e] + i * RT_ROWS;
+      tl[2] = min(RT_ROWS, c - i * RT_ROWS);
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += blockDim.x) count[e] = start[e];      // now the next free row
+  __syncthreads();
+  for (int i = tid; i < n; i += blockDim.x) {
+    const int place = atomicAdd(&count[chosen[i]], 1);
+    order[place] = i;
+    place_of[i] = place;
+  }
+}
+
+extern "C" const char* sl_route_tokens(const float* logits, int stride, int T, int E, int top, int* chosen,
+                                       float* shares, int* order, int* place_of, int* tiles, int max_tiles,
+                                       hipStream_t stream) {
+  SL_CHECK(T >= 0 && E >= 1 && E <= 4096 && top >= 1 && top <= 64 && top <= E && E <= stride,
+           "route_tokens: at most 4096 experts within the rows, at most 64 choices");
+  SL_CHECK(max_tiles >= ((long long)T * top + RT_ROWS - 1) / RT_ROWS + E, "route_tokens: too few tile entries");
+  if (T == 0) return nullptr;
+  route_kernel<<<T, 64, 0, stream>>>(logits, stride, E, top, chosen, shares);
+  group_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(chosen, T * top, E, max_tiles, order, place_of, tiles);
+  return sl_launch_status();
+}
+
+// ------------------------------------------------------------------ grouped products
+struct Grouped {
+  const act_t* x;            // row r reads x + src(r) * K, src(r) = order[r] / top when order is given, else r
+  const int* order;
+  int top;
+  const act_t* w;            // [experts][N_w][K]; gated: N_w = 2 N, gate rows before up rows
+  const int* tiles;          // [max_tiles][3]
+  int N, K;
+  act_t* out_act;            // gated: [rows][N]
+  float* out_f32;            // plain: [rows][N]
+};
+
+// 256 threads: thread (row = tid / 16, lane16 = tid % 16) owns columns lane16 + 16 u, u < 4, of a
+// 16 x 64 tile.  x and W go through LDS in chunks of 32 values of k; sums are float.
+template <bool GATED>
+__global__ __launch_bounds__(256) void grouped_product_kernel(const Grouped a) {
+  const int* tl = a.tiles + 3 * blockIdx.x;
+  const int rows = tl[2];
+  if (rows == 0) return;
+  const int e = tl[0], row0 = tl[1];
+  const int n0 = blockIdx.y * 64;
+  __shared__ float xs[RT_ROWS][33];
+  __shared__ float ws[GATED ? 128 : 64][33];
+  const int tid = threadIdx.x, r = tid / 16, l = tid % 16;
+  const size_t n_w = GATED ? 2 * (size_t)a.N : (size_t)a.N;
+  const act_t* we = a.w + (size_t)e * n_w * a.K;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f}, acc2[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < a.K; k0 += 32) {
+    __syncthreads();
+    for (int i = tid; i < RT_ROWS * 32; i += 256) {
+      const int rr = i / 32, kk = i % 32;
+      float v = 0.f;
+      if (rr < rows && k0 + kk < a.K) {
+        const size_t src = a.order != nullptr ? (size_t)(a.order[row0 + rr] / a.top) : (size_t)(row0 + rr);
+        v = to_f(a.x[src * a.K + k0 + kk]);
+      }
+      xs[rr][kk] = v;
+    }
+    for (int i = tid; i < (GATED ? 128 : 64) * 32; i += 256) {
+      const int c = i / 32, kk = i % 32;
+      const int n = n0 + (c % 64);
+      float v = 0.f;
+      if (n < a.N && k0 + kk < a.K) v = to_f(we[((size_t)(c / 64) * a.N + n) * a.K + k0 + kk]);
+      ws[c][kk] = v;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < 32; ++kk) {
+      const float xv = xs[r][kk];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        acc[u] += xv * ws[l + 16 * u][kk];
+        if (GATED) acc2[u] += xv * ws[64 + l + 16 * u][kk];
+      }
+    }
+  }
+  if (r >= rows) return;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int n = n0 + l + 16 * u;
+    if (n >= a.N) continue;
+    const size_t at = (size_t)(row0 + r) * a.N + n;
+    if (GATED) {
+      const float g = acc[u];
+      a.out_act[at] = from_f<act_t>(g / (1.f + expf(-g)) * acc2[u]);
+    } else {
+      a.out_f32[at] = acc[u];
+    }
+  }
+}
+
+extern "C" const char* sl_grouped_product(const void* x, const int* order, int top, const void* w, const int* tiles,
+                                          int max_tiles, int N, int K, int gated, void* out, hipStream_t stream) {
+  SL_CHECK(max_tiles >= 0 && N > 0 && K > 0 && top >= 1, "grouped_product: sizes must be positive");
+  if (max_tiles == 0) return nullptr;
+  const Grouped a{(const act_t*)x, order, top, (const act_t*)w, tiles, N, K, gated ? (act_t*)out : nullptr,
+                  gated ? nullptr : (float*)out};
+  const dim3 grid(max_tiles, (N + 63) / 64);
+  if (gated) grouped_product_kernel<true><<<grid, 256, 0, stream>>>(a);
+  else grouped_product_kernel<false><<<grid, 256, 0, stream>>>(a);
+  return sl_launch_status();
+}
+
+// ------------------------------------------------------------------ combine
+// out[t] = base[t] + sum_k shares[t][k] * y[place_of[t top + k]], float sums, choices in their order.
+__global__ void routed_combine_kernel(const float* __restrict__ y, const int* __restrict__ place_of,
+                                      const float* __restrict__ shares, int top, const act_t* __restrict__ base,
+                                      int H, act_t* __restrict__ out) {
+  const size_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    float v = base != nullptr ? to_f(base[t * H + c]) : 0.f;
+    for (int k = 0; k < top; ++k) v += shares[t * top + k] * y[(size_t)place_of[t * top + k] * H + c];
+    out[t * H + c] = from_f<act_t>(v);
+  }
+}
+
+extern "C" const char* sl_routed_combine(const float* y, const int* place_of, const float* shares, int T, int top,
+                                         const void* base, int H, void* out, hipStream_t stream) {
+  SL_CHECK(T >= 0 && top >= 1 && H > 0, "routed_combine: sizes must be positive");
+  if (T == 0) return nullptr;
+  routed_combine_kernel<<<T, 256, 0, stream>>>(y, place_of, shares, top, (const act_t*)base, H, (act_t*)out);
+  return sl_launch_status();
+}

@@ -173,7 +173,7 @@ def load(u: Unit) -> ctypes.CDLL:
 
 # the units every model needs; LAZY_STEMS are compiled when a model first asks for them
 DEFAULT_STEMS = ("elementwise", "norm", "gemm", "attention", "sampling")
-LAZY_STEMS = ("window_attention", "head_gemm")
+LAZY_STEMS = ("window_attention", "head_gemm", "recurrent", "routed")
 
 
 # (key width, value width, values in the key rows) the matrix-core window attention is built for

@@ -15,6 +15,7 @@ float32 table never does: its products are the hand-written float32 kernels
 from .attention_ops import AttentionOps
 from .norm_ops import NormOps
 from .product_ops import ProductOps
+from .recurrent_ops import RecurrentOps
 from .sampling_ops import SamplingOps
 from .table import KernelTable
 from .window_ops import WindowOps
@@ -22,8 +23,10 @@ from .values import (Deferred, KernelError, LinearWeight, PartialSums, RotationP
                      ScaledRows, TiledRows, _RopeStore, _c_float, _p, _ptr)
 
 
-class HipOps(NormOps, ProductOps, AttentionOps, WindowOps, SamplingOps, KernelTable):
+class HipOps(NormOps, ProductOps, AttentionOps, WindowOps, RecurrentOps, SamplingOps, KernelTable):
     """The whole table: the base (libraries, calls, checks) and one group of calls per domain.
     ``norm_ops``: embedding, add + norm, silu-multiply; ``product_ops``: weights and products;
     ``attention_ops``: rotation, cache write, attention; ``sampling_ops``: argmax and draws;
-    ``window_ops``: layer norm, per-head products, attention with a kept-first window, bias, sink and gate."""
+    ``window_ops``: layer norm, per-head products, attention with a kept-first window, bias, sink and gate;
+    ``recurrent_ops``: a norm on a sublayer's output, matrix memories in state slots (short convolution,
+    scans, read-out), attention normed over its projection, routed experts."""

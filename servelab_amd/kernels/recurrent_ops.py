@@ -1,0 +1,249 @@
+"""Calls for mixers that keep a matrix per head in a state slot, for a softmax attention whose q
+and k are normed over the whole projection, for an RMS norm on a sublayer's output, and for
+routed experts.  Their libraries (``recurrent``, ``routed``) are compiled when a model first
+asks for them.
+
+What is float32 here in both activation types: the input projections' sums as these calls read
+them, gates, decays and their logarithms, unit norms, states, read-outs, router logits and
+shares, the experts' weighted sum."""
+import ctypes
+from typing import NamedTuple
+
+import torch
+
+from .values import KernelError, _c_float, _p
+
+_ll = ctypes.c_longlong
+
+_EXPAND_MODES = {"plain": 0, "log_sigmoid": 1, "rate_softplus": 2}
+_SCAN_DECAY, _SCAN_DELTA, _SCAN_LSTM = 0, 1, 2
+_TILE_ROWS = 16               # RT_ROWS of routed.hip
+
+
+class Routing(NamedTuple):
+    """A step's routing on the device: per token the chosen experts [T, top] (int32) and their
+    shares (float32); the (token, choice) pairs sorted by expert (``order`` [T top], ``place_of``
+    its inverse) and the row tiles [max_tiles, 3] = (expert, first row, rows) the grouped
+    products walk."""
+    chosen: torch.Tensor
+    shares: torch.Tensor
+    order: torch.Tensor
+    place_of: torch.Tensor
+    tiles: torch.Tensor
+
+
+class RecurrentOps:
+    # ------------------------------------------------- norm on an output
+    def add_postnorm(self, resid, y, weight, eps, mult):
+        """resid += mult * y / sqrt(mean(y^2) + eps) * weight in place (float32); returns the
+        stream's rows in the activation dtype.  ``y`` None: only those rows."""
+        T, H = resid.shape
+        self._check(resid, torch.float32, None, "residual stream")
+        self._check(weight, torch.float32, (H,), "norm weight")
+        if y is not None:
+            self._check(y, self.act_dtype, (T, H), "sublayer output")
+        out = self._new((T, H))
+        self._call("norm", "sl_add_postnorm", _p(resid), _p(y), _p(weight), _p(out), T, H, _c_float(eps),
+                   _c_float(mult))
+        return out
+
+    def scaled_sum(self, a, sa, b, sb):
+        self._check(a, self.act_dtype, None, "a")
+        self._check(b, self.act_dtype, tuple(a.shape), "b")
+        out = self._new(tuple(a.shape))
+        self._call("norm", "sl_scaled_sum", _p(a), _c_float(sa), _p(b), _c_float(sb), _p(out), _ll(a.numel()))
+        return out
+
+    def softcap(self, logits, cap):
+        """logits <- cap * tanh(logits / cap), in place (float32)."""
+        self._check(logits, torch.float32, None, "logits")
+        self._call("norm", "sl_softcap", _p(logits), _c_float(cap), _ll(logits.numel()))
+        return logits
+
+    # ------------------------------------------------- what a scan reads
+    def _f32_rows(self, t, name):
+        self._check(t, torch.float32, None, name)
+        if t.dim() != 2:
+            raise KernelError(f"{name} must be rows [T, width]")
+        return t.shape
+
+    def _sequences(self, batch, T):
+        self._check(batch.cu_q, torch.int32, (batch.num_seqs + 1,), "cu_q")
+        self._check(batch.positions, torch.int32, (T,), "positions")
+        self._check(batch.tok_seq, torch.int32, (T,), "tok_seq")
+        self._check(batch.state_slots, torch.int32, (batch.num_seqs,), "state slots")
+        if T != batch.num_tokens:
+            raise KernelError(f"{T} rows for a batch of {batch.num_tokens} tokens")
+
+    def _state(self, state, need):
+        self._check(state, torch.float32, None, "state")
+        if state.dim() != 2 or state.shape[1] < need:
+            raise KernelError(f"state slots of {list(state.shape[1:])} values, {need} needed")
+        return state.shape[1]
+
+    def lowrank_expand(self, buf, col, w2, bias, mode, heads=1, divisor=1.0, rates=None):
+        """z = buf[:, col:col + rank] w2^T + bias as float32 [T, C]: "plain" z, "log_sigmoid"
+        logsigmoid(z) / divisor, "rate_softplus" -exp(rates[h]) softplus(z) with h = c // (C / heads)."""
+        T, stride = self._f32_rows(buf, "projected rows")
+        C, rank = w2.shape
+        self._check(w2, torch.float32, None, "expansion matrix")
+        if bias is not None:
+            self._check(bias, torch.float32, (C,), "bias")
+        if rates is not None:
+            self._check(rates, torch.float32, (heads,), "rates")
+        if mode not in _EXPAND_MODES:
+            raise KernelError(f"lowrank_expand: unknown mode {mode!r}")
+        out = self._new((T, C), torch.float32)
+        self._call(self._lazy("recurrent"), "sl_lowrank_expand", _p(buf), stride, col, rank, _p(w2), _p(bias), T, C,
+                   _EXPAND_MODES[mode], _c_float(divisor), _p(rates), heads, _p(out))
+        return out
+
+    def short_conv(self, buf, col, taps, state, state_off, batch, write, unit_heads=0, unit_dim=0,
+                   unit_eps=1e-6, scaled_heads=0, scale=1.0):
+        """silu of a causal convolution over time per channel of buf[:, col:col + C] (``taps``
+        [C, n], the last one the token's own).  The n - 1 inputs before a step come from the
+        sequence's state slot at ``state_off`` ([n - 1, C], zeros at a sequence's start), and the
+        step's last n - 1 inputs go back there.  The first ``unit_heads`` heads of ``unit_dim``
+        channels are divided by sqrt(sum x^2 + unit_eps), the first ``scaled_heads`` of them also
+        multiplied by ``scale``.  Returns float32 [T, C]."""
+        T, stride = self._f32_rows(buf, "projected rows")
+        C, n = taps.shape
+        self._check(taps, torch.float32, None, "taps")
+        self._sequences(batch, T)
+        slot_size = self._state(state, state_off + (n - 1) * C)
+        out = self._new((T, C), torch.float32)
+        self._call(self._lazy("recurrent"), "sl_short_conv", _p(buf), stride, col, C, n, _p(taps), _p(state),
+                   _ll(slot_size), state_off, _p(batch.cu_q), _p(batch.positions), _p(batch.tok_seq),
+                   _p(batch.state_slots), batch.num_seqs, T, int(bool(write)), unit_heads, unit_dim,
+                   _c_float(unit_eps), scaled_heads, _c_float(scale), _p(out))
+        return out
+
+    def _scan(self, mode, src, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, gates, i_col, f_col,
+              cap, state, batch, write):
+        T, stride = self._f32_rows(src, "q, k, v rows")
+        self._sequences(batch, T)
+        need = H * Dv * D + (H * D + H if mode == _SCAN_LSTM else 0)
+        slot_size = self._state(state, need)
+        if log_decay is not None:
+            self._check(log_decay, torch.float32, (T, H * D), "log decays")
+        gate_stride = 0
+        if gates is not None:
+            gate_stride = self._f32_rows(gates, "gates")[1]
+            if gates.shape[0] != T:
+                raise KernelError("gates for another number of tokens")
+        out = self._new((T, H * Dv), torch.float32)
+        self._call(self._lazy("recurrent"), "sl_matrix_scan", mode, _p(src), stride, q_col, k_col, v_col, H, G,
+                   D, Dv, _p(log_decay), _c_float(q_scale), _p(gates), gate_stride, i_col, f_col, _c_float(cap),
+                   _p(state), _ll(slot_size), _p(batch.cu_q), _p(batch.positions), _p(batch.state_slots),
+                   batch.num_seqs, T, int(bool(write)), _p(out))
+        return out
+
+    def decay_scan(self, src, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, beta_src, beta_col,
+                   state, batch, write):
+        """Per head S' = diag(exp(log_decay)) S + k v^T, o = S'^T (q_scale q); with ``beta_src``
+        (float32 rows holding beta before its sigmoid at column ``beta_col`` + head) the delta rule:
+        S' = diag(..) S, u = sigmoid(beta) (v - S'^T k), S' += k u^T.  q and k have G heads in
+        ``src`` (head h reads h // (H / G)).  The slot holds S as [H, Dv, D] from 0 on; a sequence
+        whose first token is in the step starts from zero.  Returns float32 [T, H Dv]."""
+        if beta_src is None:
+            return self._scan(_SCAN_DECAY, src, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, None,
+                              0, 0, 1.0, state, batch, write)
+        return self._scan(_SCAN_DELTA, src, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, beta_src,
+                          beta_col, 0, 1.0, state, batch, write)
+
+    def mlstm_scan(self, buf, q_col, k_col, v_col, i_col, f_col, H, D, Dv, cap, q_scale, state, batch, write):
+        """The matrix LSTM: i = cap tanh(i~ / cap), f = logsigmoid(cap tanh(f~ / cap)), m' = max(f + m, i),
+        S' = e^(f + m - m') S + e^(i - m') k v^T, n' likewise with k; returns S'^T q / (max(|n' . q|,
+        e^-m') + 1e-6) as float32 [T, H Dv].  The slot holds S [H, Dv, D], n [H, D], m [H]; m starts at 0."""
+        return self._scan(_SCAN_LSTM, buf, q_col, k_col, v_col, H, H, D, Dv, None, q_scale, buf, i_col, f_col,
+                          cap, state, batch, write)
+
+    def head_norm_gate(self, o, H, Dv, weight, per_head, eps, gate, gate_col, activation):
+        """Each head of ``o`` [T, H Dv] (float32) divided by its root mean square, times ``weight``
+        ([H Dv] when ``per_head``, else [Dv] for every head), times sigmoid or silu of
+        gate[:, gate_col + h Dv + d] (float32 rows).  Returns rows in the activation dtype."""
+        T, width = self._f32_rows(o, "read-out")
+        if width != H * Dv:
+            raise KernelError("head_norm_gate: the read-out is not [T, heads * channels]")
+        self._check(weight, torch.float32, (H * Dv if per_head else Dv,), "gain")
+        gate_stride = self._f32_rows(gate, "gates")[1]
+        if gate.shape[0] != T or activation not in ("sigmoid", "silu"):
+            raise KernelError("head_norm_gate: gates for another number of tokens, or an unknown activation")
+        out = self._new((T, H * Dv))
+        self._call(self._lazy("recurrent"), "sl_head_norm_gate", _p(o), T, H, Dv, _p(weight), int(bool(per_head)),
+                   _c_float(eps), _p(gate), gate_stride, gate_col, 0 if activation == "sigmoid" else 1, _p(out))
+        return out
+
+    # ------------------------------- attention: norm over the projection, rotation, pages
+    def projnorm_rope_store(self, buf, H, G, D, Dv, q_gain, k_gain, eps, rot, tables, slots, k_cache, v_cache,
+                            page_size):
+        """``buf`` (float32) holds q [H D], k [G D] and v [G Dv] side by side.  q and k are
+        RMS-normed over all their heads at once (gains of that size), the first ``rot`` channels of
+        every head rotated in halves by ``tables``; k and v go to the token's place in the pages
+        (``slots`` None: no write); q comes back as [T, H D] in the activation dtype."""
+        T, stride = self._f32_rows(buf, "projected rows")
+        self._check(q_gain, torch.float32, (H * D,), "q gain")
+        self._check(k_gain, torch.float32, (G * D,), "k gain")
+        cos = sin = None
+        if rot:
+            cos, sin = tables.cos, tables.sin
+            self._check(cos, torch.float32, (T, rot // 2), "cos")
+            self._check(sin, torch.float32, (T, rot // 2), "sin")
+        if slots is not None:
+            pages = k_cache.shape[0]
+            self._check(k_cache, self.act_dtype, (pages, G, page_size, D), "K pages")
+            self._check(v_cache, self.act_dtype, (pages, G, Dv, page_size), "V pages")
+            self._check(slots, torch.int32, (T,), "slots")
+        q = self._new((T, H * D))
+        self._call(self._lazy("recurrent"), "sl_projnorm_rope_store", _p(buf), stride, T, H, G, D, Dv, _p(q_gain),
+                   _p(k_gain), _c_float(eps), rot, _p(cos), _p(sin), _p(slots),
+                   _p(k_cache) if slots is not None else None, _p(v_cache) if slots is not None else None,
+                   page_size, _p(q))
+        return q
+
+    # ------------------------------------------------------- routed experts
+    def route_tokens(self, logits, experts, top):
+        """The ``top`` largest of each row's first ``experts`` logits (float32; among equals the
+        lower index) with the softmax over them, and the step's (token, choice) pairs sorted by
+        expert for the grouped products."""
+        T, stride = self._f32_rows(logits, "router logits")
+        n = T * top
+        max_tiles = -(-n // _TILE_ROWS) + experts
+        chosen = self._new((T, top), torch.int32)
+        shares = self._new((T, top), torch.float32)
+        order = self._new((n,), torch.int32)
+        place_of = self._new((n,), torch.int32)
+        tiles = self._new((max_tiles, 3), torch.int32)
+        self._call(self._lazy("routed"), "sl_route_tokens", _p(logits), stride, T, experts, top, _p(chosen),
+                   _p(shares), _p(order), _p(place_of), _p(tiles), max_tiles)
+        return Routing(chosen, shares, order, place_of, tiles)
+
+    def routed_experts(self, x, routing, w_gate_up, w_down, base=None):
+        """sum over a token's choices of share * down_e(silu(gate_e x) * up_e x), plus ``base``;
+        ``w_gate_up`` [E, 2 ff, width] holds an expert's gate rows before its up rows, ``w_down``
+        [E, width, ff].  Sums are float32; what lies between the two products is rounded to the
+        activation dtype."""
+        T, K = x.shape
+        E, two_ff, K2 = w_gate_up.shape
+        ff = two_ff // 2
+        self._check(x, self.act_dtype, None, "x")
+        self._check(w_gate_up, self.act_dtype, (E, 2 * ff, K), "gate/up matrices")
+        self._check(w_down, self.act_dtype, (E, K, ff), "down matrices")
+        top = routing.chosen.shape[1]
+        n = T * top
+        max_tiles = routing.tiles.shape[0]
+        if routing.chosen.shape[0] != T or max_tiles < -(-n // _TILE_ROWS) + E:
+            raise KernelError("routed_experts: the routing is for another step or other experts")
+        if base is not None:
+            self._check(base, self.act_dtype, (T, K), "base")
+        lib = self._lazy("routed")
+        mid = self._new((n, ff))
+        self._call(lib, "sl_grouped_product", _p(x), _p(routing.order), top, _p(w_gate_up), _p(routing.tiles),
+                   max_tiles, ff, K, 1, _p(mid))
+        y = self._new((n, K), torch.float32)
+        self._call(lib, "sl_grouped_product", _p(mid), None, 1, _p(w_down), _p(routing.tiles), max_tiles, K, ff,
+                   0, _p(y))
+        out = self._new((T, K))
+        self._call(lib, "sl_routed_combine", _p(y), _p(routing.place_of), _p(routing.shares), T, top, _p(base), K,
+                   _p(out))
+        return out
