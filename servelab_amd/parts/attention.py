@@ -148,7 +148,7 @@ class ProjectionNormAttention(Mixer):
         self.b_in = self.b_o = None
         if self.bias:
             b = torch.cat([tensors(n["q_bias"]).float(), tensors(n["k_bias"]).float(),
-                           tensors(n["v_bias"]).float(), torch.zeros(extra)], 0)
+                           tensors(n["v_bias"]).float(), torch.zeros(extra, device=w.device)], 0)
             self.b_in = rt.vector(b)
             self.b_o = rt.vector(tensors(n["out_bias"]))
         self.q_gain = rt.vector(tensors(n["q_norm"]))

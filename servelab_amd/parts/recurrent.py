@@ -54,7 +54,7 @@ class _MatrixMemoryMixer(Mixer):
         self.w_in = rt.linear_weight(w)
         self.b_in = None
         if biases:
-            b = torch.zeros(w.shape[0], dtype=torch.float32)
+            b = torch.zeros(w.shape[0], dtype=torch.float32, device=w.device)
             for name, t in biases.items():
                 b[self.at[name]:self.at[name] + t.shape[0]] = t.float()
             self.b_in = rt.vector(b)
