@@ -86,9 +86,49 @@ def design_configs(shape, layers, window, keep_first=4, kv_rank=512, rot_dim=64)
     return topelorn, qwen
 
 
+# Layer sizes for --design vekanex: a real model's width, heads and feed-forward; the experts' sizes are
+# such that a token's experts (top of them plus the shared one) have the dense feed-forward's width.
+VEKANEX_SHAPES = {
+    "3b": dict(memory_heads=8, memory_dim=128, memory_vdim=256, experts=64, top=8, expert_ff=1024, shared_ff=2816),
+    "7b": dict(memory_heads=14, memory_dim=128, memory_vdim=256, experts=64, top=8, expert_ff=1792, shared_ff=4608),
+}
+
+
+def vekanex_configs(shape, layers):
+    """(Vekanex config.json, Qwen2 config.json) of equal size: layers in the order matrix LSTM, softmax
+    attention beside a gated delta rule, gated linear attention, and the first layer's weights once more;
+    the attention has Qwen2's heads, every layer routed experts whose active width is Qwen2's feed-forward."""
+    z, v = DESIGN_SHAPES[shape], VEKANEX_SHAPES[shape]
+    assert v["top"] * v["expert_ff"] + v["shared_ff"] == z["ff"]
+    mlp = {"kind": "moe", "router": {"experts": v["experts"], "top": v["top"]}, "expert": {"ff": v["expert_ff"]},
+           "shared": {"ff": v["shared_ff"]}}
+    H, D, Dv = v["memory_heads"], v["memory_dim"], v["memory_vdim"]
+    mlstm = {"type": "mlstm", "mlp": mlp, "mixer": {"heads": H, "dim": D, "vdim": Dv, "gate_cap": 15.0}}
+    gla = {"type": "gla", "mlp": mlp, "mixer": {"heads": H, "dim": D, "vdim": Dv, "tau": 16.0, "decay_rank": 16}}
+    both = {"type": "parallel", "mlp": mlp, "mixer": {
+        "left": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                 "scale": z["dim"] ** -0.5, "rot": {"base": 1e6, "dims": z["dim"] // 2}},
+        "right": {"heads": 2 * H, "kv_heads": H, "dim": D, "vdim": Dv // 2, "conv": 4, "decay_rank": 32,
+                  "gate_rank": 32},
+        "left_scale": 1.0, "right_scale": 1.0}}
+    order = [mlstm, both, gla, dict(mlstm, weights_of=0)]
+    listed = []
+    for i in range(layers):
+        entry = order[i % 4]
+        if "weights_of" in entry:
+            entry = dict(entry, weights_of=i - 3)
+        listed.append(entry)
+    vekanex = {"architecture": "Vekanex", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-5},
+               "residual_mult": 0.5, "logit_softcap": 30.0, "torch_dtype": "bfloat16", "layers": listed}
+    qwen = dict(QWEN25_7B, num_hidden_layers=layers, hidden_size=z["width"], num_attention_heads=z["heads"],
+                num_key_value_heads=z["kv_heads"], head_dim=z["dim"], intermediate_size=z["ff"],
+                vocab_size=z["vocab"], tie_word_embeddings=False, use_sliding_window=False)
+    return vekanex, qwen
+
+
 def compare_designs(args):
-    """Prefill and decode throughput of the Topelorn design beside the Qwen2 decoder of equal size, at
-    each of --design-shapes: one JSON line, tokens per second each."""
+    """Prefill and decode throughput of the design named by --design beside the Qwen2 decoder of equal
+    size, at each of --design-shapes: one JSON line, tokens per second each."""
     import torch
     import servelab_amd  # noqa: F401
     from servelab_amd.config import resolve_architecture
@@ -101,7 +141,9 @@ def compare_designs(args):
                       "prefill_chunk": args.prefill_chunk, "page_size": page}, "shapes": {}}
     for shape in args.design_shapes.split(","):
         row = {}
-        for name, raw in zip(("topelorn", "qwen2"), design_configs(shape, args.design_layers, args.design_window)):
+        pair = vekanex_configs(shape, args.design_layers) if args.design == "vekanex" else \
+            design_configs(shape, args.design_layers, args.design_window)
+        for name, raw in zip((args.design, "qwen2"), pair):
             cfg = resolve_architecture(raw).config_from_hf(raw, "")
             model = random_model_on_device(cfg, args.seed, args.dtype, "cuda:0")
             torch.cuda.synchronize()
@@ -112,8 +154,8 @@ def compare_designs(args):
                          "prefill_tok_s": round(args.prefill_tokens / pre_s, 1), "prefill_ms": round(pre_s * 1e3, 3)}
             del model
             torch.cuda.empty_cache()
-        row["decode_ratio"] = round(row["topelorn"]["decode_tok_s"] / row["qwen2"]["decode_tok_s"], 3)
-        row["prefill_ratio"] = round(row["topelorn"]["prefill_tok_s"] / row["qwen2"]["prefill_tok_s"], 3)
+        row["decode_ratio"] = round(row[args.design]["decode_tok_s"] / row["qwen2"]["decode_tok_s"], 3)
+        row["prefill_ratio"] = round(row[args.design]["prefill_tok_s"] / row["qwen2"]["prefill_tok_s"], 3)
         out["shapes"][shape] = row
     print(json.dumps(out))
     return 0
@@ -266,7 +308,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernel choice for the prompt products")
-    ap.add_argument("--design", default="", choices=["", "topelorn"],
+    ap.add_argument("--design", default="", choices=["", "topelorn", "vekanex"],
                     help="instead of the default workload: prefill and decode throughput of this design "
                          "beside the Qwen2 decoder of equal size")
     ap.add_argument("--design-shapes", default="3b,7b", help="comma-separated: " + ", ".join(sorted(DESIGN_SHAPES)))

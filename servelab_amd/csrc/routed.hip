@@ -15,7 +15,7 @@
 // list of launches that a captured graph can replay.
 #include "common.h"
 
-#define RT_ROWS 16           // rows of a tile of the grouped products
+#define RT_ROWS 16           // rows of a tile of the plain grouped product; a row tile holds 16 or 64 rows
 
 // ------------------------------------------------------------------ route
 // One wavefront per token.  Largest first; among equal logits the lower index wins.
@@ -66,8 +66,8 @@ __global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ log
 //   order[place] = pair (token * top + choice);  place_of[pair] = place
 //   tiles[i] = {expert, first row, rows} for i < tiles in use; rows 0 beyond
 __global__ __launch_bounds__(1024) void group_kernel(const int* __restrict__ chosen, int n, int E, int max_tiles,
-                                                     int* __restrict__ order, int* __restrict__ place_of,
-                                                     int* __restrict__ tiles) {
+                                                     int tile_rows, int* __restrict__ order,
+                                                     int* __restrict__ place_of, int* __restrict__ tiles) {
   extern __shared__ int sh[];
   int* count = sh;               // [E]
   int* start = sh + E;           // [E] first row of the expert
@@ -88,17 +88,17 @@ __global__ __launch_bounds__(1024) void group_kernel(const int* __restrict__ cho
       start[e] = rows;
       tile0[e] = nt;
       rows += count[e];
-      nt += (count[e] + RT_ROWS - 1) / RT_ROWS;
+      nt += (count[e] + tile_rows - 1) / tile_rows;
     }
   }
   __syncthreads();
   for (int e = tid; e < E; e += blockDim.x) {
     const int c = count[e];
-    for (int i = 0; i * RT_ROWS < c; ++i) {
+    for (int i = 0; i * tile_rows < c; ++i) {
       int* tl = tiles + 3 * (tile0[e] + i);
       tl[0] = e;
-      tl[1] = start[e] + i * RT_ROWS;
-      tl[2] = min(RT_ROWS, c - i * RT_ROWS);
+      tl[1] = start[e] + i * tile_rows;
+      tl[2] = min(tile_rows, c - i * tile_rows);
     }
   }
   __syncthreads();
@@ -113,13 +113,15 @@ __global__ __launch_bounds__(1024) void group_kernel(const int* __restrict__ cho
 
 extern "C" const char* sl_route_tokens(const float* logits, int stride, int T, int E, int top, int* chosen,
                                        float* shares, int* order, int* place_of, int* tiles, int max_tiles,
-                                       hipStream_t stream) {
+                                       int tile_rows, hipStream_t stream) {
   SL_CHECK(T >= 0 && E >= 1 && E <= 4096 && top >= 1 && top <= 64 && top <= E && E <= stride,
            "route_tokens: at most 4096 experts within the rows, at most 64 choices");
-  SL_CHECK(max_tiles >= ((long long)T * top + RT_ROWS - 1) / RT_ROWS + E, "route_tokens: too few tile entries");
+  SL_CHECK(tile_rows == 16 || tile_rows == 64, "route_tokens: row tiles hold 16 or 64 rows");
+  SL_CHECK(max_tiles >= ((long long)T * top + tile_rows - 1) / tile_rows + E, "route_tokens: too few tile entries");
   if (T == 0) return nullptr;
   route_kernel<<<T, 64, 0, stream>>>(logits, stride, E, top, chosen, shares);
-  group_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(chosen, T * top, E, max_tiles, order, place_of, tiles);
+  group_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(chosen, T * top, E, max_tiles, tile_rows, order, place_of,
+                                                         tiles);
   return sl_launch_status();
 }
 
@@ -130,6 +132,7 @@ struct Grouped {
   int top;
   const act_t* w;            // [experts][N_w][K]; gated: N_w = 2 N, gate rows before up rows
   const int* tiles;          // [max_tiles][3]
+  int sub;                   // row tiles hold 16 * sub rows
   int N, K;
   act_t* out_act;            // gated: [rows][N]
   float* out_f32;            // plain: [rows][N]
@@ -139,10 +142,11 @@ struct Grouped {
 // 16 x 64 tile.  x and W go through LDS in chunks of 32 values of k; sums are float.
 template <bool GATED>
 __global__ __launch_bounds__(256) void grouped_product_kernel(const Grouped a) {
-  const int* tl = a.tiles + 3 * blockIdx.x;
-  const int rows = tl[2];
-  if (rows == 0) return;
-  const int e = tl[0], row0 = tl[1];
+  const int* tl = a.tiles + 3 * (blockIdx.x / a.sub);
+  const int part = blockIdx.x % a.sub;                  // which 16 rows of the row tile
+  const int rows = min(RT_ROWS, tl[2] - RT_ROWS * part);
+  if (rows <= 0) return;
+  const int e = tl[0], row0 = tl[1] + RT_ROWS * part;
   const int n0 = blockIdx.y * 64;
   __shared__ float xs[RT_ROWS][33];
   __shared__ float ws[GATED ? 128 : 64][33];
@@ -194,13 +198,109 @@ __global__ __launch_bounds__(256) void grouped_product_kernel(const Grouped a) {
   }
 }
 
+#if !defined(SL_F32)
+typedef __bf16 rt_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 rt_bf16x4 __attribute__((ext_vector_type(4)));
+typedef float rt_f32x4 __attribute__((ext_vector_type(4)));
+
+// The same on the matrix cores (bfloat16, K in steps of 32, N in steps of 16): a wavefront owns a
+// row tile (NT x 16 rows of one expert) by NU x 16 columns and reads its operands straight from
+// memory, eight values a lane: rows of W are the first operand of mfma 16x16x32, rows of x the
+// second; the gated form keeps gate and up sums of the same columns.  Rows past the tile's last are
+// computed like the last and never stored.
+template <int NT, int NU, bool GATED>
+__global__ __launch_bounds__(64) void grouped_product_mfma_kernel(const Grouped a) {
+  const int* tl = a.tiles + 3 * blockIdx.x;
+  const int rows = tl[2];
+  if (rows == 0) return;
+  const int e = tl[0], row0 = tl[1];
+  const int lane = threadIdx.x, i = lane & 15, gq = lane >> 4;
+  const int n0 = blockIdx.y * 16 * NU;
+  const size_t n_w = GATED ? 2 * (size_t)a.N : (size_t)a.N;
+  const __bf16* we = a.w + (size_t)e * n_w * a.K;
+  const __bf16* xp[NT];
+#pragma unroll
+  for (int v = 0; v < NT; ++v) {
+    const int rr = row0 + min(16 * v + i, rows - 1);
+    const size_t src = a.order != nullptr ? (size_t)(a.order[rr] / a.top) : (size_t)rr;
+    xp[v] = a.x + src * a.K + 8 * gq;
+  }
+  const __bf16* wp[NU];
+#pragma unroll
+  for (int u = 0; u < NU; ++u) wp[u] = we + (size_t)min(n0 + 16 * u + i, a.N - 1) * a.K + 8 * gq;
+  const size_t up = (size_t)a.N * a.K;                  // from a gate row to its up row
+  rt_f32x4 acc[NT][NU], acc2[NT][GATED ? NU : 1];
+#pragma unroll
+  for (int v = 0; v < NT; ++v)
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+      acc[v][u] = rt_f32x4{0.f, 0.f, 0.f, 0.f};
+      if (GATED) acc2[v][u] = rt_f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll 2
+  for (int k = 0; k < a.K; k += 32) {
+    rt_bf16x8 b[NT], w1[NU], w2[GATED ? NU : 1];
+#pragma unroll
+    for (int v = 0; v < NT; ++v) b[v] = *(const rt_bf16x8*)(xp[v] + k);
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+      w1[u] = *(const rt_bf16x8*)(wp[u] + k);
+      if (GATED) w2[u] = *(const rt_bf16x8*)(wp[u] + up + k);
+    }
+#pragma unroll
+    for (int v = 0; v < NT; ++v)
+#pragma unroll
+      for (int u = 0; u < NU; ++u) {
+        acc[v][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u], b[v], acc[v][u], 0, 0, 0);
+        if (GATED) acc2[v][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w2[u], b[v], acc2[v][u], 0, 0, 0);
+      }
+  }
+  // this lane holds columns n0 + 16 u + 4 gq .. + 3 of rows 16 v + i
+#pragma unroll
+  for (int v = 0; v < NT; ++v) {
+    if (16 * v + i >= rows) continue;
+    const size_t at = (size_t)(row0 + 16 * v + i) * a.N + n0 + 4 * gq;
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+      if (n0 + 16 * u >= a.N) continue;
+      if (GATED) {
+        rt_bf16x4 r;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const float g = acc[v][u][c];
+          r[c] = (__bf16)(g / (1.f + expf(-g)) * acc2[v][u][c]);
+        }
+        *(rt_bf16x4*)(a.out_act + at + 16 * u) = r;
+      } else {
+        *(rt_f32x4*)(a.out_f32 + at + 16 * u) = acc[v][u];
+      }
+    }
+  }
+}
+#endif
+
 extern "C" const char* sl_grouped_product(const void* x, const int* order, int top, const void* w, const int* tiles,
-                                          int max_tiles, int N, int K, int gated, void* out, hipStream_t stream) {
+                                          int max_tiles, int tile_rows, int N, int K, int gated, void* out,
+                                          hipStream_t stream) {
   SL_CHECK(max_tiles >= 0 && N > 0 && K > 0 && top >= 1, "grouped_product: sizes must be positive");
+  SL_CHECK(tile_rows == 16 || tile_rows == 64, "grouped_product: row tiles hold 16 or 64 rows");
   if (max_tiles == 0) return nullptr;
-  const Grouped a{(const act_t*)x, order, top, (const act_t*)w, tiles, N, K, gated ? (act_t*)out : nullptr,
-                  gated ? nullptr : (float*)out};
-  const dim3 grid(max_tiles, (N + 63) / 64);
+  const Grouped a{(const act_t*)x, order, top, (const act_t*)w, tiles, tile_rows / RT_ROWS, N, K,
+                  gated ? (act_t*)out : nullptr, gated ? nullptr : (float*)out};
+#if !defined(SL_F32)
+  if (K % 32 == 0 && N % 16 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const dim3 grid(max_tiles, (N + 63) / 64);
+    if (tile_rows == 64) {
+      if (gated) grouped_product_mfma_kernel<4, 4, true><<<grid, 64, 0, stream>>>(a);
+      else grouped_product_mfma_kernel<4, 4, false><<<grid, 64, 0, stream>>>(a);
+    } else {
+      if (gated) grouped_product_mfma_kernel<1, 4, true><<<grid, 64, 0, stream>>>(a);
+      else grouped_product_mfma_kernel<1, 4, false><<<grid, 64, 0, stream>>>(a);
+    }
+    return sl_launch_status();
+  }
+#endif
+  const dim3 grid(max_tiles * (tile_rows / RT_ROWS), (N + 63) / 64);
   if (gated) grouped_product_kernel<true><<<grid, 256, 0, stream>>>(a);
   else grouped_product_kernel<false><<<grid, 256, 0, stream>>>(a);
   return sl_launch_status();

@@ -17,22 +17,25 @@ _ll = ctypes.c_longlong
 
 _EXPAND_MODES = {"plain": 0, "log_sigmoid": 1, "rate_softplus": 2}
 _SCAN_DECAY, _SCAN_DELTA, _SCAN_LSTM = 0, 1, 2
-_TILE_ROWS = 16               # RT_ROWS of routed.hip
+_TILE_ROWS = (16, 64)         # rows of a row tile of the grouped products (routed.hip)
 
 
 class Routing(NamedTuple):
     """A step's routing on the device: per token the chosen experts [T, top] (int32) and their
     shares (float32); the (token, choice) pairs sorted by expert (``order`` [T top], ``place_of``
-    its inverse) and the row tiles [max_tiles, 3] = (expert, first row, rows) the grouped
-    products walk."""
+    its inverse) and the row tiles [max_tiles, 3] = (expert, first row, rows) of at most
+    ``tile_rows`` rows that the grouped products walk."""
     chosen: torch.Tensor
     shares: torch.Tensor
     order: torch.Tensor
     place_of: torch.Tensor
     tiles: torch.Tensor
+    tile_rows: int
 
 
 class RecurrentOps:
+    ROUTED_WIDE_TILE_ROWS = 48    # rows an expert has on average from which row tiles hold 64 rows
+
     # ------------------------------------------------- norm on an output
     def add_postnorm(self, resid, y, weight, eps, mult):
         """resid += mult * y / sqrt(mean(y^2) + eps) * weight in place (float32); returns the
@@ -208,15 +211,18 @@ class RecurrentOps:
         expert for the grouped products."""
         T, stride = self._f32_rows(logits, "router logits")
         n = T * top
-        max_tiles = -(-n // _TILE_ROWS) + experts
+        # tiles of 64 rows once an expert has that many on average: its matrices are then read
+        # once per 64 rows instead of once per 16
+        tile_rows = _TILE_ROWS[1] if n >= experts * self.ROUTED_WIDE_TILE_ROWS else _TILE_ROWS[0]
+        max_tiles = -(-n // tile_rows) + experts
         chosen = self._new((T, top), torch.int32)
         shares = self._new((T, top), torch.float32)
         order = self._new((n,), torch.int32)
         place_of = self._new((n,), torch.int32)
         tiles = self._new((max_tiles, 3), torch.int32)
         self._call(self._lazy("routed"), "sl_route_tokens", _p(logits), stride, T, experts, top, _p(chosen),
-                   _p(shares), _p(order), _p(place_of), _p(tiles), max_tiles)
-        return Routing(chosen, shares, order, place_of, tiles)
+                   _p(shares), _p(order), _p(place_of), _p(tiles), max_tiles, tile_rows)
+        return Routing(chosen, shares, order, place_of, tiles, tile_rows)
 
     def routed_experts(self, x, routing, w_gate_up, w_down, base=None):
         """sum over a token's choices of share * down_e(silu(gate_e x) * up_e x), plus ``base``;
@@ -232,17 +238,17 @@ class RecurrentOps:
         top = routing.chosen.shape[1]
         n = T * top
         max_tiles = routing.tiles.shape[0]
-        if routing.chosen.shape[0] != T or max_tiles < -(-n // _TILE_ROWS) + E:
+        if routing.chosen.shape[0] != T or max_tiles < -(-n // routing.tile_rows) + E:
             raise KernelError("routed_experts: the routing is for another step or other experts")
         if base is not None:
             self._check(base, self.act_dtype, (T, K), "base")
         lib = self._lazy("routed")
         mid = self._new((n, ff))
         self._call(lib, "sl_grouped_product", _p(x), _p(routing.order), top, _p(w_gate_up), _p(routing.tiles),
-                   max_tiles, ff, K, 1, _p(mid))
+                   max_tiles, routing.tile_rows, ff, K, 1, _p(mid))
         y = self._new((n, K), torch.float32)
-        self._call(lib, "sl_grouped_product", _p(mid), None, 1, _p(w_down), _p(routing.tiles), max_tiles, K, ff,
-                   0, _p(y))
+        self._call(lib, "sl_grouped_product", _p(mid), None, 1, _p(w_down), _p(routing.tiles), max_tiles,
+                   routing.tile_rows, K, ff, 0, _p(y))
         out = self._new((T, K))
         self._call(lib, "sl_routed_combine", _p(y), _p(routing.place_of), _p(routing.shares), T, top, _p(base), K,
                    _p(out))

@@ -217,7 +217,7 @@ def test_route_tokens_sorts_the_pairs_by_expert(T, E, top):
     covered = []
     for e, row0, rows in tiles.tolist():
         if rows:
-            assert 1 <= rows <= 16 and (by_row[row0:row0 + rows] == e).all()
+            assert 1 <= rows <= r.tile_rows and (by_row[row0:row0 + rows] == e).all()
             covered += list(range(row0, row0 + rows))
     assert covered == list(range(T * top))
 
