@@ -184,7 +184,23 @@ struct MatrixScan {
 };
 
 enum { SCAN_DECAY = 0, SCAN_DELTA = 1, SCAN_LSTM = 2 };
-#define SCAN_ROWS 8          // key channels a lane owns: channels p, p + P, ..., p + 7 P
+#define SCAN_ROWS 8          // key channels a lane owns: channels 8 p .. 8 p + 7
+
+// Sum over the P lanes that share a column (P a power of two, the lanes adjacent and aligned); every
+// lane gets the sum.  Within 16 lanes by data-parallel moves (neighbours in a quad, the other pair of
+// the quad, the mirrored half row, the mirrored row), beyond that by shuffles.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float group_sum(float v, int P) {
+  if (P >= 2) v += dpp_move<0xB1>(v);          // quad_perm [1, 0, 3, 2]
+  if (P >= 4) v += dpp_move<0x4E>(v);          // quad_perm [2, 3, 0, 1]
+  if (P >= 8) v += dpp_move<0x141>(v);         // row_half_mirror
+  if (P >= 16) v += dpp_move<0x140>(v);        // row_mirror
+  for (int w = 16; w < P; w <<= 1) v += __shfl_xor(v, w, SL_WAVE);
+  return v;
+}
+struct __attribute__((aligned(16))) scan_f4 { float v[4]; };
 
 // A block of 256 threads takes a (sequence, head, slice of value channels): P lanes share a
 // column of S (P a power of two with 8 P >= D), 256 / P columns a block.  The step's tokens go
@@ -193,15 +209,16 @@ enum { SCAN_DECAY = 0, SCAN_DELTA = 1, SCAN_LSTM = 2 };
 // column adding their parts of the read-out by butterfly.
 template <int MODE>
 __global__ __launch_bounds__(256) void matrix_scan_kernel(const MatrixScan a, int P, int CH) {
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   const int s = blockIdx.x, h = blockIdx.y, slice = blockIdx.z, tid = threadIdx.x;
   const int Dp = P * SCAN_ROWS, cols = 256 / P;
+  const int lgDp = __ffs(Dp) - 1, lgCols = __ffs(cols) - 1;
   float* sq = lds;                       // [CH][Dp]
   float* sk = sq + CH * Dp;              // [CH][Dp]
   float* sa = sk + CH * Dp;              // [CH][Dp] decays (not for the matrix LSTM)
   float* sv = MODE == SCAN_LSTM ? sa : sa + CH * Dp;     // [CH][cols]
   float* sg = sv + CH * cols;            // [CH][2] gates
-  const int p = tid % P, cl = tid / P;
+  const int p = tid & (P - 1), cl = tid >> (__ffs(P) - 1);
   const int j = slice * cols + cl;
   const bool live = j < a.Dv;
   const int g = h / (a.H / a.G);
@@ -214,71 +231,112 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(const MatrixScan a, in
   float* mcell = slot + nS + (size_t)a.H * a.D + h;
   float S[SCAN_ROWS], n[SCAN_ROWS];
   float m = 0.f;
+  const int r0 = p * SCAN_ROWS;
 #pragma unroll
   for (int i = 0; i < SCAN_ROWS; ++i) {
-    const int r = i * P + p;
+    const int r = r0 + i;
     S[i] = (!fresh && live && r < a.D) ? col[r] : 0.f;
     n[i] = (MODE == SCAN_LSTM && !fresh && r < a.D) ? nrow[r] : 0.f;
   }
   if (MODE == SCAN_LSTM && !fresh) m = *mcell;
 
-  for (int t0 = first; t0 < last; t0 += CH) {
-    const int nt = min(CH, last - t0);
-    __syncthreads();
-    for (int idx = tid; idx < nt * Dp; idx += 256) {
-      const int tt = idx / Dp, r = idx % Dp;
-      const size_t t = t0 + tt;
-      float q = 0.f, k = 0.f, d = 1.f;
-      if (r < a.D) {
-        q = a.src[t * a.src_stride + a.q_col + g * a.D + r] * a.q_scale;
-        k = a.src[t * a.src_stride + a.k_col + g * a.D + r];
-        if (MODE != SCAN_LSTM) d = expf(a.log_decay[(t * a.H + h) * a.D + r]);
+  // A chunk's inputs are asked for a chunk ahead and wait in registers while the chunk before is
+  // walked: at most 8 values of q, k and the decays and 8 of v a thread (the host keeps CH within that).
+  float pq[8], pk[8], pd[8], pv[8], pg0 = 0.f, pg1 = 0.f;
+  auto fetch = [&](int t0, int nt) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int idx = tid + e * 256;
+      pq[e] = 0.f;
+      pk[e] = 0.f;
+      pd[e] = 0.f;
+      pv[e] = 0.f;
+      if (idx < nt * Dp) {
+        const int tt = idx >> lgDp, r = idx & (Dp - 1);            // (Dp and cols are powers of two)
+        const size_t t = t0 + tt;
+        if (r < a.D) {
+          pq[e] = a.src[t * a.src_stride + a.q_col + g * a.D + r] * a.q_scale;
+          pk[e] = a.src[t * a.src_stride + a.k_col + g * a.D + r];
+          if (MODE != SCAN_LSTM) pd[e] = a.log_decay[(t * a.H + h) * a.D + r];
+        }
       }
-      sq[idx] = q;
-      sk[idx] = k;
-      if (MODE != SCAN_LSTM) sa[idx] = d;
-    }
-    for (int idx = tid; idx < nt * cols; idx += 256) {
-      const int tt = idx / cols, c = slice * cols + idx % cols;
-      sv[idx] = c < a.Dv ? a.src[(size_t)(t0 + tt) * a.src_stride + a.v_col + h * a.Dv + c] : 0.f;
+      if (idx < nt * cols) {
+        const int tt = idx >> lgCols, c = slice * cols + (idx & (cols - 1));
+        if (c < a.Dv) pv[e] = a.src[(size_t)(t0 + tt) * a.src_stride + a.v_col + h * a.Dv + c];
+      }
     }
     if (MODE != SCAN_DECAY && tid < nt) {
       const float* gr = a.gates + (size_t)(t0 + tid) * a.gate_stride;
+      pg0 = gr[a.i_col + h];
+      if (MODE == SCAN_LSTM) pg1 = gr[a.f_col + h];
+    }
+  };
+  fetch(first, min(CH, last - first));
+  for (int t0 = first; t0 < last; t0 += CH) {
+    const int nt = min(CH, last - t0);
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int idx = tid + e * 256;
+      if (idx < nt * Dp) {
+        sq[idx] = pq[e];
+        sk[idx] = pk[e];
+        if (MODE != SCAN_LSTM) sa[idx] = expf(pd[e]);
+      }
+      if (idx < nt * cols) sv[idx] = pv[e];
+    }
+    if (MODE != SCAN_DECAY && tid < nt) {
       if (MODE == SCAN_DELTA) {
-        sg[tid * 2] = sigmoidf_(gr[a.i_col + h]);
+        sg[tid * 2] = sigmoidf_(pg0);
       } else {
-        sg[tid * 2] = a.cap * tanhf(gr[a.i_col + h] / a.cap);
-        sg[tid * 2 + 1] = logsigmoidf_(a.cap * tanhf(gr[a.f_col + h] / a.cap));
+        sg[tid * 2] = a.cap * tanhf(pg0 / a.cap);
+        sg[tid * 2 + 1] = logsigmoidf_(a.cap * tanhf(pg1 / a.cap));
       }
     }
     __syncthreads();
+    if (t0 + CH < last) fetch(t0 + CH, min(CH, last - t0 - CH));
+#pragma unroll 2
     for (int tt = 0; tt < nt; ++tt) {
-      const float* q = sq + tt * Dp;
-      const float* k = sk + tt * Dp;
-      const float* d = sa + tt * Dp;
+      float q[SCAN_ROWS], k[SCAN_ROWS], d[SCAN_ROWS];
+      {
+        const scan_f4* q4 = (const scan_f4*)(sq + tt * Dp + r0);
+        const scan_f4* k4 = (const scan_f4*)(sk + tt * Dp + r0);
+        const scan_f4* d4 = (const scan_f4*)(sa + tt * Dp + r0);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const scan_f4 qv = q4[u], kv = k4[u];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            q[4 * u + c] = qv.v[c];
+            k[4 * u + c] = kv.v[c];
+          }
+          if (MODE != SCAN_LSTM) {
+            const scan_f4 dv = d4[u];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) d[4 * u + c] = dv.v[c];
+          }
+        }
+      }
       const float v = sv[tt * cols + cl];
       float o = 0.f, aux = 0.f;
       if (MODE == SCAN_DECAY) {
 #pragma unroll
         for (int i = 0; i < SCAN_ROWS; ++i) {
-          const int r = i * P + p;
-          S[i] = d[r] * S[i] + k[r] * v;
-          o += S[i] * q[r];
+          S[i] = d[i] * S[i] + k[i] * v;
+          o += S[i] * q[i];
         }
       } else if (MODE == SCAN_DELTA) {
 #pragma unroll
         for (int i = 0; i < SCAN_ROWS; ++i) {
-          const int r = i * P + p;
-          S[i] *= d[r];
-          aux += S[i] * k[r];
+          S[i] *= d[i];
+          aux += S[i] * k[i];
         }
-        for (int w = 1; w < P; w <<= 1) aux += __shfl_xor(aux, w, SL_WAVE);
+        aux = group_sum(aux, P);
         const float u = sg[tt * 2] * (v - aux);
 #pragma unroll
         for (int i = 0; i < SCAN_ROWS; ++i) {
-          const int r = i * P + p;
-          S[i] += k[r] * u;
-          o += S[i] * q[r];
+          S[i] += k[i] * u;
+          o += S[i] * q[i];
         }
       } else {
         const float ig = sg[tt * 2], fg = sg[tt * 2 + 1];
@@ -287,17 +345,16 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(const MatrixScan a, in
         m = top;
 #pragma unroll
         for (int i = 0; i < SCAN_ROWS; ++i) {
-          const int r = i * P + p;
-          const float ak = add * k[r];
+          const float ak = add * k[i];
           S[i] = keep * S[i] + ak * v;
           n[i] = keep * n[i] + ak;
-          o += S[i] * q[r];
-          aux += n[i] * q[r];
+          o += S[i] * q[i];
+          aux += n[i] * q[i];
         }
       }
-      for (int w = 1; w < P; w <<= 1) o += __shfl_xor(o, w, SL_WAVE);
+      o = group_sum(o, P);
       if (MODE == SCAN_LSTM) {
-        for (int w = 1; w < P; w <<= 1) aux += __shfl_xor(aux, w, SL_WAVE);
+        aux = group_sum(aux, P);
         o = o / (fmaxf(fabsf(aux), expf(-m)) + 1e-6f);
       }
       if (p == 0 && live) a.out[((size_t)(t0 + tt) * a.H + h) * a.Dv + j] = o;
@@ -306,7 +363,7 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(const MatrixScan a, in
   if (a.write) {
 #pragma unroll
     for (int i = 0; i < SCAN_ROWS; ++i) {
-      const int r = i * P + p;
+      const int r = r0 + i;
       if (live && r < a.D) col[r] = S[i];
       if (MODE == SCAN_LSTM && slice == 0 && cl == 0 && r < a.D) nrow[r] = n[i];
     }
@@ -335,7 +392,7 @@ extern "C" const char* sl_matrix_scan(int mode, const float* src, int src_stride
   int P = 1;
   while (P * SCAN_ROWS < D) P <<= 1;
   const int cols = 256 / P, Dp = P * SCAN_ROWS;
-  const int CH = Dp <= 128 ? 16 : (Dp <= 256 ? 8 : 4);
+  const int CH = min(Dp <= 128 ? 16 : (Dp <= 256 ? 8 : 4), 8 * P);     // 8 values a thread of each kind a chunk
   const size_t lds = (size_t)CH * ((mode == SCAN_LSTM ? 2 : 3) * Dp + cols + 2) * sizeof(float);
   const MatrixScan a{src, src_stride, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, gates, gate_stride,
                      i_col, f_col, cap, state, state_stride, cu_q, positions, slots, write, out};

@@ -15,7 +15,7 @@
 // list of launches that a captured graph can replay.
 #include "common.h"
 
-#define RT_ROWS 16           // rows of a tile of the plain grouped product; a row tile holds 16 or 64 rows
+#define RT_ROWS 16           // rows of a tile of the plain grouped product; a row tile holds 16, 64 or 128 rows
 
 // ------------------------------------------------------------------ route
 // One wavefront per token.  Largest first; among equal logits the lower index wins.
@@ -116,7 +116,7 @@ extern "C" const char* sl_route_tokens(const float* logits, int stride, int T, i
                                        int tile_rows, hipStream_t stream) {
   SL_CHECK(T >= 0 && E >= 1 && E <= 4096 && top >= 1 && top <= 64 && top <= E && E <= stride,
            "route_tokens: at most 4096 experts within the rows, at most 64 choices");
-  SL_CHECK(tile_rows == 16 || tile_rows == 64, "route_tokens: row tiles hold 16 or 64 rows");
+  SL_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "route_tokens: row tiles hold 16, 64 or 128 rows");
   SL_CHECK(max_tiles >= ((long long)T * top + tile_rows - 1) / tile_rows + E, "route_tokens: too few tile entries");
   if (T == 0) return nullptr;
   route_kernel<<<T, 64, 0, stream>>>(logits, stride, E, top, chosen, shares);
@@ -203,19 +203,22 @@ typedef __bf16 rt_bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 rt_bf16x4 __attribute__((ext_vector_type(4)));
 typedef float rt_f32x4 __attribute__((ext_vector_type(4)));
 
-// The same on the matrix cores (bfloat16, K in steps of 32, N in steps of 16): a wavefront owns a
-// row tile (NT x 16 rows of one expert) by NU x 16 columns and reads its operands straight from
+// The same on the matrix cores (bfloat16, K in steps of 32, N in steps of 16): a wavefront owns
+// NT x 16 rows of a row tile by NU x 16 columns and reads its operands straight from
 // memory, eight values a lane: rows of W are the first operand of mfma 16x16x32, rows of x the
 // second; the gated form keeps gate and up sums of the same columns.  Rows past the tile's last are
 // computed like the last and never stored.
-template <int NT, int NU, bool GATED>
-__global__ __launch_bounds__(64) void grouped_product_mfma_kernel(const Grouped a) {
+template <int NT, int NU, bool GATED, int WR, int WC>
+__global__ __launch_bounds__(64 * WR * WC) void grouped_product_mfma_kernel(const Grouped a) {
+  // WR x WC wavefronts a workgroup: WR along the rows of the row tile, WC along the columns; those
+  // that read the same rows of x or of W find them in the CU's cache after the first has asked
   const int* tl = a.tiles + 3 * blockIdx.x;
-  const int rows = tl[2];
-  if (rows == 0) return;
-  const int e = tl[0], row0 = tl[1];
-  const int lane = threadIdx.x, i = lane & 15, gq = lane >> 4;
-  const int n0 = blockIdx.y * 16 * NU;
+  const int wave = threadIdx.x / 64, wr = wave % WR, wc = wave / WR;
+  const int rows = min(16 * NT, tl[2] - 16 * NT * wr);
+  const int n0 = (blockIdx.y * WC + wc) * 16 * NU;
+  if (rows <= 0 || n0 >= a.N) return;
+  const int e = tl[0], row0 = tl[1] + 16 * NT * wr;
+  const int lane = threadIdx.x & 63, i = lane & 15, gq = lane >> 4;
   const size_t n_w = GATED ? 2 * (size_t)a.N : (size_t)a.N;
   const __bf16* we = a.w + (size_t)e * n_w * a.K;
   const __bf16* xp[NT];
@@ -283,19 +286,24 @@ extern "C" const char* sl_grouped_product(const void* x, const int* order, int t
                                           int max_tiles, int tile_rows, int N, int K, int gated, void* out,
                                           hipStream_t stream) {
   SL_CHECK(max_tiles >= 0 && N > 0 && K > 0 && top >= 1, "grouped_product: sizes must be positive");
-  SL_CHECK(tile_rows == 16 || tile_rows == 64, "grouped_product: row tiles hold 16 or 64 rows");
+  SL_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "grouped_product: row tiles hold 16, 64 or 128 rows");
   if (max_tiles == 0) return nullptr;
   const Grouped a{(const act_t*)x, order, top, (const act_t*)w, tiles, tile_rows / RT_ROWS, N, K,
                   gated ? (act_t*)out : nullptr, gated ? nullptr : (float*)out};
 #if !defined(SL_F32)
   if (K % 32 == 0 && N % 16 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0) {
-    const dim3 grid(max_tiles, (N + 63) / 64);
-    if (tile_rows == 64) {
-      if (gated) grouped_product_mfma_kernel<4, 4, true><<<grid, 64, 0, stream>>>(a);
-      else grouped_product_mfma_kernel<4, 4, false><<<grid, 64, 0, stream>>>(a);
+    if (tile_rows == 128) {                             // two wavefronts along the rows, two along the columns
+      const dim3 grid(max_tiles, (N + 127) / 128);
+      if (gated) grouped_product_mfma_kernel<4, 4, true, 2, 2><<<grid, 256, 0, stream>>>(a);
+      else grouped_product_mfma_kernel<4, 4, false, 2, 2><<<grid, 256, 0, stream>>>(a);
+    } else if (tile_rows == 64) {
+      const dim3 grid(max_tiles, (N + 255) / 256);
+      if (gated) grouped_product_mfma_kernel<4, 4, true, 1, 4><<<grid, 256, 0, stream>>>(a);
+      else grouped_product_mfma_kernel<4, 4, false, 1, 4><<<grid, 256, 0, stream>>>(a);
     } else {
-      if (gated) grouped_product_mfma_kernel<1, 4, true><<<grid, 64, 0, stream>>>(a);
-      else grouped_product_mfma_kernel<1, 4, false><<<grid, 64, 0, stream>>>(a);
+      const dim3 grid(max_tiles, (N + 63) / 64);
+      if (gated) grouped_product_mfma_kernel<1, 4, true, 1, 1><<<grid, 64, 0, stream>>>(a);
+      else grouped_product_mfma_kernel<1, 4, false, 1, 1><<<grid, 64, 0, stream>>>(a);
     }
     return sl_launch_status();
   }
@@ -308,21 +316,31 @@ extern "C" const char* sl_grouped_product(const void* x, const int* order, int t
 
 // ------------------------------------------------------------------ combine
 // out[t] = base[t] + sum_k shares[t][k] * y[place_of[t top + k]], float sums, choices in their order.
-__global__ void routed_combine_kernel(const float* __restrict__ y, const int* __restrict__ place_of,
-                                      const float* __restrict__ shares, int top, const act_t* __restrict__ base,
-                                      int H, act_t* __restrict__ out) {
+__global__ __launch_bounds__(256) void routed_combine_kernel(const float* __restrict__ y,
+                                                             const int* __restrict__ place_of,
+                                                             const float* __restrict__ shares, int top,
+                                                             const act_t* __restrict__ base, int H,
+                                                             act_t* __restrict__ out) {
+  __shared__ int place[64];
+  __shared__ float share[64];
   const size_t t = blockIdx.x;
-  for (int c = threadIdx.x; c < H; c += blockDim.x) {
-    float v = base != nullptr ? to_f(base[t * H + c]) : 0.f;
-    for (int k = 0; k < top; ++k) v += shares[t * top + k] * y[(size_t)place_of[t * top + k] * H + c];
-    out[t * H + c] = from_f<act_t>(v);
+  if (threadIdx.x < top) {
+    place[threadIdx.x] = place_of[t * top + threadIdx.x];
+    share[threadIdx.x] = shares[t * top + threadIdx.x];
   }
+  __syncthreads();
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= H) return;
+  float v = base != nullptr ? to_f(base[t * H + c]) : 0.f;
+  for (int k = 0; k < top; ++k) v += share[k] * y[(size_t)place[k] * H + c];
+  out[t * H + c] = from_f<act_t>(v);
 }
 
 extern "C" const char* sl_routed_combine(const float* y, const int* place_of, const float* shares, int T, int top,
                                          const void* base, int H, void* out, hipStream_t stream) {
-  SL_CHECK(T >= 0 && top >= 1 && H > 0, "routed_combine: sizes must be positive");
+  SL_CHECK(T >= 0 && top >= 1 && top <= 64 && H > 0, "routed_combine: sizes must be positive, at most 64 choices");
   if (T == 0) return nullptr;
-  routed_combine_kernel<<<T, 256, 0, stream>>>(y, place_of, shares, top, (const act_t*)base, H, (act_t*)out);
+  routed_combine_kernel<<<dim3(T, (H + 255) / 256), 256, 0, stream>>>(y, place_of, shares, top, (const act_t*)base, H,
+                                                                    (act_t*)out);
   return sl_launch_status();
 }

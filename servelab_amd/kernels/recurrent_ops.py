@@ -17,7 +17,7 @@ _ll = ctypes.c_longlong
 
 _EXPAND_MODES = {"plain": 0, "log_sigmoid": 1, "rate_softplus": 2}
 _SCAN_DECAY, _SCAN_DELTA, _SCAN_LSTM = 0, 1, 2
-_TILE_ROWS = (16, 64)         # rows of a row tile of the grouped products (routed.hip)
+_TILE_ROWS = (16, 64, 128)    # rows of a row tile of the grouped products (routed.hip)
 
 
 class Routing(NamedTuple):
@@ -211,9 +211,11 @@ class RecurrentOps:
         expert for the grouped products."""
         T, stride = self._f32_rows(logits, "router logits")
         n = T * top
-        # tiles of 64 rows once an expert has that many on average: its matrices are then read
-        # once per 64 rows instead of once per 16
-        tile_rows = _TILE_ROWS[1] if n >= experts * self.ROUTED_WIDE_TILE_ROWS else _TILE_ROWS[0]
+        # larger row tiles once an expert has that many rows on average: its matrices are then read
+        # once per 64 or 128 rows instead of once per 16
+        per_expert = n / experts
+        tile_rows = _TILE_ROWS[2] if per_expert >= 2 * self.ROUTED_WIDE_TILE_ROWS else \
+            (_TILE_ROWS[1] if per_expert >= self.ROUTED_WIDE_TILE_ROWS else _TILE_ROWS[0])
         max_tiles = -(-n // tile_rows) + experts
         chosen = self._new((T, top), torch.int32)
         shares = self._new((T, top), torch.float32)
