@@ -232,10 +232,20 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(const MatrixScan a, in
   float S[SCAN_ROWS], n[SCAN_ROWS];
   float m = 0.f;
   const int r0 = p * SCAN_ROWS;
+  // (a lane's 8 values of a column are one 32-byte piece where the slot's place allows it)
+  const bool whole = live && r0 + SCAN_ROWS <= a.D && ((uintptr_t)(col + r0) % 16) == 0;
+  if (whole && !fresh) {
+    const scan_f4 lo = ((const scan_f4*)(col + r0))[0], hi = ((const scan_f4*)(col + r0))[1];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      S[c] = lo.v[c];
+      S[4 + c] = hi.v[c];
+    }
+  }
 #pragma unroll
   for (int i = 0; i < SCAN_ROWS; ++i) {
     const int r = r0 + i;
-    S[i] = (!fresh && live && r < a.D) ? col[r] : 0.f;
+    if (!(whole && !fresh)) S[i] = (!fresh && live && r < a.D) ? col[r] : 0.f;
     n[i] = (MODE == SCAN_LSTM && !fresh && r < a.D) ? nrow[r] : 0.f;
   }
   if (MODE == SCAN_LSTM && !fresh) m = *mcell;
@@ -361,10 +371,20 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(const MatrixScan a, in
     }
   }
   if (a.write) {
+    if (whole) {
+      scan_f4 lo, hi;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        lo.v[c] = S[c];
+        hi.v[c] = S[4 + c];
+      }
+      ((scan_f4*)(col + r0))[0] = lo;
+      ((scan_f4*)(col + r0))[1] = hi;
+    }
 #pragma unroll
     for (int i = 0; i < SCAN_ROWS; ++i) {
       const int r = r0 + i;
-      if (live && r < a.D) col[r] = S[i];
+      if (!whole && live && r < a.D) col[r] = S[i];
       if (MODE == SCAN_LSTM && slice == 0 && cl == 0 && r < a.D) nrow[r] = n[i];
     }
     if (MODE == SCAN_LSTM && slice == 0 && tid == 0) *mcell = m;

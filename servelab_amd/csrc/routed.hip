@@ -240,7 +240,7 @@ __global__ __launch_bounds__(64 * WR * WC) void grouped_product_mfma_kernel(cons
       acc[v][u] = rt_f32x4{0.f, 0.f, 0.f, 0.f};
       if (GATED) acc2[v][u] = rt_f32x4{0.f, 0.f, 0.f, 0.f};
     }
-#pragma unroll 2
+#pragma unroll 4
   for (int k = 0; k < a.K; k += 32) {
     rt_bf16x8 b[NT], w1[NU], w2[GATED ? NU : 1];
 #pragma unroll
