@@ -131,6 +131,8 @@ struct Grouped {
   const int* order;
   int top;
   const act_t* w;            // [experts][N_w][K]; gated: N_w = 2 N, gate rows before up rows
+  int w_tiled;               // an expert's matrix lies as [N_w / 16][K / 32][64 lanes][8], lane = 16 (k / 8 % 4) + n % 16:
+                             // the first operand of mfma 16x16x32 as it sits in registers, 1 KB a wavefront's load
   const int* tiles;          // [max_tiles][3]
   int sub;                   // row tiles hold 16 * sub rows
   int N, K;
@@ -229,9 +231,13 @@ __global__ __launch_bounds__(64 * WR * WC) void grouped_product_mfma_kernel(cons
     xp[v] = a.x + src * a.K + 8 * gq;
   }
   const __bf16* wp[NU];
+  const int wstep = a.w_tiled ? 512 : 32;               // elements from one k-step to the next
 #pragma unroll
-  for (int u = 0; u < NU; ++u) wp[u] = we + (size_t)min(n0 + 16 * u + i, a.N - 1) * a.K + 8 * gq;
-  const size_t up = (size_t)a.N * a.K;                  // from a gate row to its up row
+  for (int u = 0; u < NU; ++u) {
+    if (a.w_tiled) wp[u] = we + (size_t)(min(n0 + 16 * u, a.N - 16) / 16) * (a.K / 32) * 512 + lane * 8;
+    else wp[u] = we + (size_t)min(n0 + 16 * u + i, a.N - 1) * a.K + 8 * gq;
+  }
+  const size_t up = (size_t)a.N * a.K;                  // from a gate row to its up row (N in steps of 16)
   rt_f32x4 acc[NT][NU], acc2[NT][GATED ? NU : 1];
 #pragma unroll
   for (int v = 0; v < NT; ++v)
@@ -243,12 +249,13 @@ __global__ __launch_bounds__(64 * WR * WC) void grouped_product_mfma_kernel(cons
 #pragma unroll 4
   for (int k = 0; k < a.K; k += 32) {
     rt_bf16x8 b[NT], w1[NU], w2[GATED ? NU : 1];
+    const size_t kw = (size_t)(k / 32) * wstep;
 #pragma unroll
     for (int v = 0; v < NT; ++v) b[v] = *(const rt_bf16x8*)(xp[v] + k);
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
-      w1[u] = *(const rt_bf16x8*)(wp[u] + k);
-      if (GATED) w2[u] = *(const rt_bf16x8*)(wp[u] + up + k);
+      w1[u] = *(const rt_bf16x8*)(wp[u] + kw);
+      if (GATED) w2[u] = *(const rt_bf16x8*)(wp[u] + up + kw);
     }
 #pragma unroll
     for (int v = 0; v < NT; ++v)
@@ -283,14 +290,17 @@ __global__ __launch_bounds__(64 * WR * WC) void grouped_product_mfma_kernel(cons
 #endif
 
 extern "C" const char* sl_grouped_product(const void* x, const int* order, int top, const void* w, const int* tiles,
-                                          int max_tiles, int tile_rows, int N, int K, int gated, void* out,
-                                          hipStream_t stream) {
+                                          int w_tiled, int max_tiles, int tile_rows, int N, int K, int gated,
+                                          void* out, hipStream_t stream) {
   SL_CHECK(max_tiles >= 0 && N > 0 && K > 0 && top >= 1, "grouped_product: sizes must be positive");
   SL_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "grouped_product: row tiles hold 16, 64 or 128 rows");
   if (max_tiles == 0) return nullptr;
-  const Grouped a{(const act_t*)x, order, top, (const act_t*)w, tiles, tile_rows / RT_ROWS, N, K,
+  const Grouped a{(const act_t*)x, order, top, (const act_t*)w, w_tiled, tiles, tile_rows / RT_ROWS, N, K,
                   gated ? (act_t*)out : nullptr, gated ? nullptr : (float*)out};
 #if !defined(SL_F32)
+#if defined(SL_F32)
+  SL_CHECK(!w_tiled, "grouped_product: tiled matrices are for bfloat16");
+#endif
   if (K % 32 == 0 && N % 16 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0) {
     if (tile_rows == 128) {                             // two wavefronts along the rows, two along the columns
       const dim3 grid(max_tiles, (N + 127) / 128);
@@ -308,6 +318,7 @@ extern "C" const char* sl_grouped_product(const void* x, const int* order, int t
     return sl_launch_status();
   }
 #endif
+  SL_CHECK(!w_tiled, "grouped_product: tiled matrices need K in steps of 32, N in steps of 16 and aligned operands");
   const dim3 grid(max_tiles * (tile_rows / RT_ROWS), (N + 63) / 64);
   if (gated) grouped_product_kernel<true><<<grid, 256, 0, stream>>>(a);
   else grouped_product_kernel<false><<<grid, 256, 0, stream>>>(a);

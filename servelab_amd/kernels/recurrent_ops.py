@@ -33,6 +33,16 @@ class Routing(NamedTuple):
     tile_rows: int
 
 
+class ExpertMatrices:
+    """The stacked matrices [E, N, K] of a set of experts as the grouped products read them:
+    row-major, or (bfloat16, N in steps of 16, K in steps of 32) every expert's matrix in the tiled
+    layout of the few-rows products, in which a wavefront's load is 1 KB of consecutive memory."""
+    __slots__ = ("data", "shape", "tiled")
+
+    def __init__(self, data, shape, tiled):
+        self.data, self.shape, self.tiled = data, tuple(shape), bool(tiled)
+
+
 class RecurrentOps:
     ROUTED_WIDE_TILE_ROWS = 48    # rows an expert has on average from which row tiles hold 64 rows
 
@@ -226,17 +236,38 @@ class RecurrentOps:
                    _p(shares), _p(order), _p(place_of), _p(tiles), max_tiles, tile_rows)
         return Routing(chosen, shares, order, place_of, tiles, tile_rows)
 
+    def prepare_expert_matrices(self, w, gated=False):
+        """Called once per stack of expert matrices [E, N, K] at load: what ``routed_experts`` takes.
+        ``gated``: the stack holds every expert's gate rows before its up rows."""
+        E, N, K = w.shape
+        self._check(w, self.act_dtype, None, "expert matrices")
+        if self.act_dtype != torch.bfloat16 or (N // 2 if gated else N) % 16 or K % 32:
+            return ExpertMatrices(w, w.shape, False)
+        tiled = torch.empty((E, N * K), dtype=torch.bfloat16, device=self.device)
+        for e in range(E):
+            self._call("gemm", "sl_tile_weight", _p(w[e]), _p(tiled[e]), N, K, 16)
+        return ExpertMatrices(tiled, w.shape, True)
+
     def routed_experts(self, x, routing, w_gate_up, w_down, base=None):
         """sum over a token's choices of share * down_e(silu(gate_e x) * up_e x), plus ``base``;
         ``w_gate_up`` [E, 2 ff, width] holds an expert's gate rows before its up rows, ``w_down``
         [E, width, ff].  Sums are float32; what lies between the two products is rounded to the
         activation dtype."""
+        if not isinstance(w_gate_up, ExpertMatrices):
+            w_gate_up = ExpertMatrices(w_gate_up, w_gate_up.shape, False)
+        if not isinstance(w_down, ExpertMatrices):
+            w_down = ExpertMatrices(w_down, w_down.shape, False)
         T, K = x.shape
         E, two_ff, K2 = w_gate_up.shape
         ff = two_ff // 2
         self._check(x, self.act_dtype, None, "x")
-        self._check(w_gate_up, self.act_dtype, (E, 2 * ff, K), "gate/up matrices")
-        self._check(w_down, self.act_dtype, (E, K, ff), "down matrices")
+        if w_gate_up.shape != (E, 2 * ff, K) or w_down.shape != (E, K, ff):
+            raise KernelError(f"routed_experts: matrices of {list(w_gate_up.shape)} and {list(w_down.shape)} "
+                              f"for rows of {K} values")
+        for m in (w_gate_up, w_down):
+            self._check(m.data, self.act_dtype, None, "expert matrices")
+            if m.data.numel() != E * m.shape[1] * m.shape[2]:
+                raise KernelError("routed_experts: expert matrices of another size than they say")
         top = routing.chosen.shape[1]
         n = T * top
         max_tiles = routing.tiles.shape[0]
@@ -246,11 +277,11 @@ class RecurrentOps:
             self._check(base, self.act_dtype, (T, K), "base")
         lib = self._lazy("routed")
         mid = self._new((n, ff))
-        self._call(lib, "sl_grouped_product", _p(x), _p(routing.order), top, _p(w_gate_up), _p(routing.tiles),
-                   max_tiles, routing.tile_rows, ff, K, 1, _p(mid))
+        self._call(lib, "sl_grouped_product", _p(x), _p(routing.order), top, _p(w_gate_up.data),
+                   _p(routing.tiles), int(w_gate_up.tiled), max_tiles, routing.tile_rows, ff, K, 1, _p(mid))
         y = self._new((n, K), torch.float32)
-        self._call(lib, "sl_grouped_product", _p(mid), None, 1, _p(w_down), _p(routing.tiles), max_tiles,
-                   routing.tile_rows, K, ff, 0, _p(y))
+        self._call(lib, "sl_grouped_product", _p(mid), None, 1, _p(w_down.data), _p(routing.tiles),
+                   int(w_down.tiled), max_tiles, routing.tile_rows, K, ff, 0, _p(y))
         out = self._new((T, K))
         self._call(lib, "sl_routed_combine", _p(y), _p(routing.place_of), _p(routing.shares), T, top, _p(base), K,
                    _p(out))

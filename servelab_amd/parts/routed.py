@@ -55,8 +55,9 @@ class RoutedExperts(FeedForward):
             p = n["expert"].format(e)
             gate_up.append(torch.cat([tensors(p + n["gate"]), tensors(p + n["up"])], 0))
             down.append(tensors(p + n["down"]))
-        self.w_gate_up = rt.matrix(torch.stack(gate_up))          # [E, 2 ff, width]
-        self.w_down = rt.matrix(torch.stack(down))                # [E, width, ff]
+        prepare = getattr(rt.ops, "prepare_expert_matrices", lambda w, gated=False: w)   # (the kernel table's layout)
+        self.w_gate_up = prepare(rt.matrix(torch.stack(gate_up)), gated=True)            # [E, 2 ff, width]
+        self.w_down = prepare(rt.matrix(torch.stack(down)))                 # [E, width, ff]
         if self.shared is not None:
             self.shared.load(prefixed(n["shared"], tensors), rt)
 

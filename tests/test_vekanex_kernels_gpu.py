@@ -238,3 +238,7 @@ def test_routed_experts(dtype, T, E, top, ff, K):
         got = hip.routed_experts(x.to(DEV), r, wgu.to(DEV), wd.to(DEV), None if b is None else b.to(DEV))
         want = emu.routed_experts(x, (r.chosen.cpu(), r.shares.cpu()), wgu, wd, b)
         close(got, want, 3e-6 if dtype == torch.float32 else 1.2e-2)
+        tiled = (hip.prepare_expert_matrices(wgu.to(DEV), gated=True), hip.prepare_expert_matrices(wd.to(DEV)))
+        assert tiled[0].tiled == (dtype == torch.bfloat16 and ff % 16 == 0 and K % 32 == 0)
+        again = hip.routed_experts(x.to(DEV), r, tiled[0], tiled[1], None if b is None else b.to(DEV))
+        assert torch.equal(again, got)                    # the same sums in the same order, from another layout
