@@ -184,7 +184,7 @@ struct MatrixScan {
 };
 
 enum { SCAN_DECAY = 0, SCAN_DELTA = 1, SCAN_LSTM = 2 };
-#define SCAN_ROWS 8          // key channels a lane owns: channels 8 p .. 8 p + 7
+constexpr int SCAN_ROWS = 8;      // key channels a lane owns: channels 8 p .. 8 p + 7
 
 // Sum over the P lanes that share a column (P a power of two, the lanes adjacent and aligned); every
 // lane gets the sum.  Within 16 lanes by data-parallel moves (neighbours in a quad, the other pair of
@@ -201,193 +201,252 @@ __device__ __forceinline__ float group_sum(float v, int P) {
   return v;
 }
 struct __attribute__((aligned(16))) scan_f4 { float v[4]; };
+template <int ROWS> __device__ __forceinline__ float rows_sum(const float* x) {
+  float s = (x[0] + x[1]) + (x[2] + x[3]);
+  if (ROWS == 8) s += (x[4] + x[5]) + (x[6] + x[7]);
+  return s;
+}
 
-// A block of 256 threads takes a (sequence, head, slice of value channels): P lanes share a
-// column of S (P a power of two with 8 P >= D), 256 / P columns a block.  The step's tokens go
-// through LDS a chunk at a time (q, k, decay of the head, v of the block's columns, gates); the
-// columns then walk the chunk token by token, a lane updating its 8 rows and the P lanes of a
-// column adding their parts of the read-out by butterfly.
-template <int MODE>
-__global__ __launch_bounds__(256) void matrix_scan_kernel(const MatrixScan a, int P, int CH) {
+
+// A block takes a (sequence, head, slice of value channels).  Its first four wavefronts walk the
+// tokens: P lanes share a column of S (P a power of two with 8 P >= D), 256 / P columns a block, a
+// lane updating its 8 rows and the P lanes of a column adding their parts of the read-out by
+// butterfly.  Its other four wavefronts bring the step's tokens into LDS a chunk ahead (q, k, the
+// decays after their exponential, v of the block's columns, the gates after their squashing), into
+// the half of LDS that the walkers are not reading; one barrier a chunk hands the halves over.  What
+// does not depend on S is done by the bringers: the matrix LSTM's running maximum and the three
+// factors a token takes from it are a scan over scalars, which one of their wavefronts carries; and
+// the walkers leave their read-outs in LDS, from where the bringers write a chunk's to memory.
+template <int MODE, int ROWS>
+__global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, int P, int CH) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  const int s = blockIdx.x, h = blockIdx.y, slice = blockIdx.z, tid = threadIdx.x;
-  const int Dp = P * SCAN_ROWS, cols = 256 / P;
+  const int s = blockIdx.x, h = blockIdx.y, slice = blockIdx.z;
+  const bool walker = threadIdx.x < 256;
+  const int tid = threadIdx.x & 255;
+  const int Dp = P * ROWS, cols = 256 / P;
   const int lgDp = __ffs(Dp) - 1, lgCols = __ffs(cols) - 1;
-  float* sq = lds;                       // [CH][Dp]
-  float* sk = sq + CH * Dp;              // [CH][Dp]
-  float* sa = sk + CH * Dp;              // [CH][Dp] decays (not for the matrix LSTM)
-  float* sv = MODE == SCAN_LSTM ? sa : sa + CH * Dp;     // [CH][cols]
-  float* sg = sv + CH * cols;            // [CH][2] gates
-  const int p = tid & (P - 1), cl = tid >> (__ffs(P) - 1);
-  const int j = slice * cols + cl;
-  const bool live = j < a.Dv;
+  const int half = CH * ((MODE == SCAN_LSTM ? 2 : 3) * Dp + 2 * cols + 4);
+  const int oq = 0, ok = CH * Dp, oa = 2 * CH * Dp;          // [CH][Dp] each (no decays for the matrix LSTM)
+  const int ov = MODE == SCAN_LSTM ? oa : oa + CH * Dp;       // [CH][cols]
+  const int og = ov + CH * cols;                              // [CH][4] gates
+  const int oo = og + CH * 4;                                 // [CH][cols] the walkers' read-outs
   const int g = h / (a.H / a.G);
   const int first = a.cu_q[s], last = a.cu_q[s + 1];
   const bool fresh = a.positions[first] == 0;
   float* slot = a.state + (size_t)a.slots[s] * a.state_stride;
-  float* col = slot + ((size_t)h * a.Dv + (live ? j : 0)) * a.D;
   const size_t nS = (size_t)a.H * a.Dv * a.D;
   float* nrow = slot + nS + (size_t)h * a.D;
   float* mcell = slot + nS + (size_t)a.H * a.D + h;
-  float S[SCAN_ROWS], n[SCAN_ROWS];
-  float m = 0.f;
-  const int r0 = p * SCAN_ROWS;
-  // (a lane's 8 values of a column are one 32-byte piece where the slot's place allows it)
-  const bool whole = live && r0 + SCAN_ROWS <= a.D && ((uintptr_t)(col + r0) % 16) == 0;
-  if (whole && !fresh) {
-    const scan_f4 lo = ((const scan_f4*)(col + r0))[0], hi = ((const scan_f4*)(col + r0))[1];
+
+  if (!walker) {
+    float m = (MODE == SCAN_LSTM && !fresh) ? *mcell : 0.f;
+    // A chunk's inputs are asked for a round ahead and wait in registers while the walkers finish the
+    // chunk before: at most 8 values of q, k and the decays and 8 of v a thread (the host keeps CH
+    // within that).
+    float pq[8], pk[8], pd[8], pv[8], g0 = 0.f, g1 = 0.f;
+    auto ask = [&](int t0, int nt) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      S[c] = lo.v[c];
-      S[4 + c] = hi.v[c];
+      for (int e = 0; e < 8; ++e) {
+        const int idx = tid + e * 256;
+        pq[e] = 0.f;
+        pk[e] = 0.f;
+        pd[e] = 0.f;
+        pv[e] = 0.f;
+        if (idx < nt * Dp) {
+          const int tt = idx >> lgDp, r = idx & (Dp - 1);          // (Dp and cols are powers of two)
+          const size_t t = t0 + tt;
+          if (r < a.D) {
+            pq[e] = a.src[t * a.src_stride + a.q_col + g * a.D + r] * a.q_scale;
+            pk[e] = a.src[t * a.src_stride + a.k_col + g * a.D + r];
+            if (MODE != SCAN_LSTM) pd[e] = a.log_decay[(t * a.H + h) * a.D + r];
+          }
+        }
+        if (idx < nt * cols) {
+          const int tt = idx >> lgCols, cc = slice * cols + (idx & (cols - 1));
+          if (cc < a.Dv) pv[e] = a.src[(size_t)(t0 + tt) * a.src_stride + a.v_col + h * a.Dv + cc];
+        }
+      }
+      if (MODE != SCAN_DECAY && tid < 64 && tid < nt) {
+        const float* gr = a.gates + (size_t)(t0 + tid) * a.gate_stride;
+        g0 = gr[a.i_col + h];
+        if (MODE == SCAN_LSTM) g1 = gr[a.f_col + h];
+      }
+    };
+    // the read-outs of chunk c - 2 lie in the half that round c fills: they leave for memory first
+    auto flush = [&](int c, int t0) {
+      if (c < 2) return;
+      const float* so = lds + (c & 1) * half + oo;
+      const int tf = t0 - 2 * CH, nf = min(CH, last - tf);
+      for (int idx = tid; idx < nf * cols; idx += 256) {
+        const int jj = slice * cols + (idx & (cols - 1));
+        if (jj < a.Dv) a.out[((size_t)(tf + (idx >> lgCols)) * a.H + h) * a.Dv + jj] = so[idx];
+      }
+    };
+    ask(first, min(CH, last - first));
+    for (int t0 = first, c = 0; t0 < last + CH; t0 += CH, ++c) {
+      // round c brings chunk c while the walkers read chunk c - 1; the last round brings nothing
+      const int nt = min(CH, last - t0);
+      flush(c, t0);
+      if (nt > 0) {
+        float* base = lds + (c & 1) * half;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int idx = tid + e * 256;
+          if (idx < nt * Dp) {
+            // channel r = ROWS p + 4 u + c of a token lies at u * 4 P + 4 p + c: the 16-byte pieces that
+            // the lanes of a column read together are then side by side and take every LDS bank once
+            const int r = idx & (Dp - 1);
+            const int at = (idx - r) + ((r & (ROWS - 1)) >> 2) * 4 * P + (r / ROWS) * 4 + (r & 3);
+            base[oq + at] = pq[e];
+            base[ok + at] = pk[e];
+            if (MODE != SCAN_LSTM) base[oa + at] = expf(pd[e]);
+          }
+          if (idx < nt * cols) base[ov + idx] = pv[e];
+        }
+        if (MODE == SCAN_DELTA && tid < nt) base[og + tid * 4] = sigmoidf_(g0);
+        if (MODE == SCAN_LSTM && tid < 64) {
+          // (CH is at most 16: the chunk's gates sit in the first lanes of this wavefront)
+          const float ig = a.cap * tanhf(g0 / a.cap), fg = logsigmoidf_(a.cap * tanhf(g1 / a.cap));
+          // the running maximum is the only chain; a lane keeps its token's two values of it and
+          // takes the exponentials afterwards, all tokens at once
+          float before = 0.f, top = 0.f;
+          for (int tt = 0; tt < nt; ++tt) {
+            const float reach = fmaxf(__shfl(fg, tt, SL_WAVE) + m, __shfl(ig, tt, SL_WAVE));
+            if (tid == tt) {
+              before = m;
+              top = reach;
+            }
+            m = reach;
+          }
+          const float keep = expf(fg + before - top), add = expf(ig - top), floor_ = expf(-top);
+          if (tid < nt) {
+            base[og + tid * 4] = keep;
+            base[og + tid * 4 + 1] = add;
+            base[og + tid * 4 + 2] = floor_;
+          }
+        }
+      }
+      if (t0 + CH < last) ask(t0 + CH, min(CH, last - t0 - CH));
+      __syncthreads();
+    }
+    {
+      const int rounds = (last - first + CH - 1) / CH + 1;
+      flush(rounds, first + rounds * CH);
+    }
+    if (MODE == SCAN_LSTM && a.write && slice == 0 && tid == 0) *mcell = m;
+    return;
+  }
+
+  const int p = tid & (P - 1), cl = tid >> (__ffs(P) - 1);
+  const int j = slice * cols + cl;
+  const bool live = j < a.Dv;
+  float* col = slot + ((size_t)h * a.Dv + (live ? j : 0)) * a.D;
+  float S[ROWS], n[ROWS];
+  const int r0 = p * ROWS;
+  // (a lane's values of a column are 16-byte pieces where the slot's place allows it)
+  const bool whole = live && r0 + ROWS <= a.D && ((uintptr_t)(col + r0) % 16) == 0;
+  if (whole && !fresh) {
+#pragma unroll
+    for (int u = 0; u < ROWS / 4; ++u) {
+      const scan_f4 piece = ((const scan_f4*)(col + r0))[u];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) S[4 * u + c] = piece.v[c];
     }
   }
 #pragma unroll
-  for (int i = 0; i < SCAN_ROWS; ++i) {
+  for (int i = 0; i < ROWS; ++i) {
     const int r = r0 + i;
     if (!(whole && !fresh)) S[i] = (!fresh && live && r < a.D) ? col[r] : 0.f;
     n[i] = (MODE == SCAN_LSTM && !fresh && r < a.D) ? nrow[r] : 0.f;
   }
-  if (MODE == SCAN_LSTM && !fresh) m = *mcell;
-
-  // A chunk's inputs are asked for a chunk ahead and wait in registers while the chunk before is
-  // walked: at most 8 values of q, k and the decays and 8 of v a thread (the host keeps CH within that).
-  float pq[8], pk[8], pd[8], pv[8], pg0 = 0.f, pg1 = 0.f;
-  auto fetch = [&](int t0, int nt) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int idx = tid + e * 256;
-      pq[e] = 0.f;
-      pk[e] = 0.f;
-      pd[e] = 0.f;
-      pv[e] = 0.f;
-      if (idx < nt * Dp) {
-        const int tt = idx >> lgDp, r = idx & (Dp - 1);            // (Dp and cols are powers of two)
-        const size_t t = t0 + tt;
-        if (r < a.D) {
-          pq[e] = a.src[t * a.src_stride + a.q_col + g * a.D + r] * a.q_scale;
-          pk[e] = a.src[t * a.src_stride + a.k_col + g * a.D + r];
-          if (MODE != SCAN_LSTM) pd[e] = a.log_decay[(t * a.H + h) * a.D + r];
-        }
-      }
-      if (idx < nt * cols) {
-        const int tt = idx >> lgCols, c = slice * cols + (idx & (cols - 1));
-        if (c < a.Dv) pv[e] = a.src[(size_t)(t0 + tt) * a.src_stride + a.v_col + h * a.Dv + c];
-      }
-    }
-    if (MODE != SCAN_DECAY && tid < nt) {
-      const float* gr = a.gates + (size_t)(t0 + tid) * a.gate_stride;
-      pg0 = gr[a.i_col + h];
-      if (MODE == SCAN_LSTM) pg1 = gr[a.f_col + h];
-    }
-  };
-  fetch(first, min(CH, last - first));
-  for (int t0 = first; t0 < last; t0 += CH) {
+  __syncthreads();                        // chunk 0 is in LDS
+  for (int t0 = first, c = 0; t0 < last; t0 += CH, ++c) {
     const int nt = min(CH, last - t0);
-    __syncthreads();
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int idx = tid + e * 256;
-      if (idx < nt * Dp) {
-        sq[idx] = pq[e];
-        sk[idx] = pk[e];
-        if (MODE != SCAN_LSTM) sa[idx] = expf(pd[e]);
-      }
-      if (idx < nt * cols) sv[idx] = pv[e];
-    }
-    if (MODE != SCAN_DECAY && tid < nt) {
-      if (MODE == SCAN_DELTA) {
-        sg[tid * 2] = sigmoidf_(pg0);
-      } else {
-        sg[tid * 2] = a.cap * tanhf(pg0 / a.cap);
-        sg[tid * 2 + 1] = logsigmoidf_(a.cap * tanhf(pg1 / a.cap));
-      }
-    }
-    __syncthreads();
-    if (t0 + CH < last) fetch(t0 + CH, min(CH, last - t0 - CH));
-#pragma unroll 2
+    float* base = lds + (c & 1) * half;
+    const float *sq = base + oq, *sk = base + ok, *sa = base + oa, *sv = base + ov, *sg = base + og;
+    float* so = base + oo;
+#pragma unroll 4
     for (int tt = 0; tt < nt; ++tt) {
-      float q[SCAN_ROWS], k[SCAN_ROWS], d[SCAN_ROWS];
+      float q[ROWS], k[ROWS], d[ROWS];
       {
-        const scan_f4* q4 = (const scan_f4*)(sq + tt * Dp + r0);
-        const scan_f4* k4 = (const scan_f4*)(sk + tt * Dp + r0);
-        const scan_f4* d4 = (const scan_f4*)(sa + tt * Dp + r0);
+        const scan_f4* q4 = (const scan_f4*)(sq + tt * Dp + 4 * p);
+        const scan_f4* k4 = (const scan_f4*)(sk + tt * Dp + 4 * p);
+        const scan_f4* d4 = (const scan_f4*)(sa + tt * Dp + 4 * p);
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const scan_f4 qv = q4[u], kv = k4[u];
+        for (int u = 0; u < ROWS / 4; ++u) {
+          const scan_f4 qv = q4[u * P], kv = k4[u * P];
 #pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            q[4 * u + c] = qv.v[c];
-            k[4 * u + c] = kv.v[c];
+          for (int c2 = 0; c2 < 4; ++c2) {
+            q[4 * u + c2] = qv.v[c2];
+            k[4 * u + c2] = kv.v[c2];
           }
           if (MODE != SCAN_LSTM) {
-            const scan_f4 dv = d4[u];
+            const scan_f4 dv = d4[u * P];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) d[4 * u + c] = dv.v[c];
+            for (int c2 = 0; c2 < 4; ++c2) d[4 * u + c2] = dv.v[c2];
           }
         }
       }
       const float v = sv[tt * cols + cl];
-      float o = 0.f, aux = 0.f;
+      float o, floor_ = 0.f;
+      float part[ROWS];
       if (MODE == SCAN_DECAY) {
 #pragma unroll
-        for (int i = 0; i < SCAN_ROWS; ++i) {
+        for (int i = 0; i < ROWS; ++i) {
           S[i] = d[i] * S[i] + k[i] * v;
-          o += S[i] * q[i];
+          part[i] = S[i] * q[i];
         }
       } else if (MODE == SCAN_DELTA) {
+        // S'^T k with S' = diag(d) S, as a sum of S (d k): the products d k do not wait for S
+        float dk[ROWS];
 #pragma unroll
-        for (int i = 0; i < SCAN_ROWS; ++i) {
-          S[i] *= d[i];
-          aux += S[i] * k[i];
-        }
-        aux = group_sum(aux, P);
-        const float u = sg[tt * 2] * (v - aux);
+        for (int i = 0; i < ROWS; ++i) dk[i] = d[i] * k[i];
 #pragma unroll
-        for (int i = 0; i < SCAN_ROWS; ++i) {
-          S[i] += k[i] * u;
-          o += S[i] * q[i];
+        for (int i = 0; i < ROWS; ++i) part[i] = S[i] * dk[i];
+        const float seen = group_sum(rows_sum<ROWS>(part), P);
+        const float u = sg[tt * 4] * (v - seen);
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) {
+          S[i] = d[i] * S[i] + k[i] * u;
+          part[i] = S[i] * q[i];
         }
       } else {
-        const float ig = sg[tt * 2], fg = sg[tt * 2 + 1];
-        const float top = fmaxf(fg + m, ig);
-        const float keep = expf(fg + m - top), add = expf(ig - top);
-        m = top;
+        const float keep = sg[tt * 4], add = sg[tt * 4 + 1];
+        floor_ = sg[tt * 4 + 2];
+        float npart[ROWS];
 #pragma unroll
-        for (int i = 0; i < SCAN_ROWS; ++i) {
+        for (int i = 0; i < ROWS; ++i) {
           const float ak = add * k[i];
           S[i] = keep * S[i] + ak * v;
           n[i] = keep * n[i] + ak;
-          o += S[i] * q[i];
-          aux += n[i] * q[i];
+          part[i] = S[i] * q[i];
+          npart[i] = n[i] * q[i];
         }
+        const float nq = group_sum(rows_sum<ROWS>(npart), P);
+        floor_ = fmaxf(fabsf(nq), floor_) + 1e-6f;
       }
-      o = group_sum(o, P);
-      if (MODE == SCAN_LSTM) {
-        aux = group_sum(aux, P);
-        o = o / (fmaxf(fabsf(aux), expf(-m)) + 1e-6f);
-      }
-      if (p == 0 && live) a.out[((size_t)(t0 + tt) * a.H + h) * a.Dv + j] = o;
+      o = group_sum(rows_sum<ROWS>(part), P);
+      if (MODE == SCAN_LSTM) o = o / floor_;
+      if (p == 0) so[tt * cols + cl] = o;
     }
+    __syncthreads();                      // chunk c + 1 is in LDS, chunk c's half is free
   }
   if (a.write) {
     if (whole) {
-      scan_f4 lo, hi;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        lo.v[c] = S[c];
-        hi.v[c] = S[4 + c];
+      for (int u = 0; u < ROWS / 4; ++u) {
+        scan_f4 piece;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) piece.v[c] = S[4 * u + c];
+        ((scan_f4*)(col + r0))[u] = piece;
       }
-      ((scan_f4*)(col + r0))[0] = lo;
-      ((scan_f4*)(col + r0))[1] = hi;
     }
 #pragma unroll
-    for (int i = 0; i < SCAN_ROWS; ++i) {
+    for (int i = 0; i < ROWS; ++i) {
       const int r = r0 + i;
       if (!whole && live && r < a.D) col[r] = S[i];
       if (MODE == SCAN_LSTM && slice == 0 && cl == 0 && r < a.D) nrow[r] = n[i];
     }
-    if (MODE == SCAN_LSTM && slice == 0 && tid == 0) *mcell = m;
   }
 }
 
@@ -409,17 +468,20 @@ extern "C" const char* sl_matrix_scan(int mode, const float* src, int src_stride
   const long long need = (long long)H * Dv * D + (mode == SCAN_LSTM ? (long long)H * D + H : 0);
   SL_CHECK(need <= state_stride, "matrix_scan: the state does not fit its slot");
   if (S == 0 || T == 0) return nullptr;
+  // (A lane owning 4 key channels instead of 8 doubles the blocks of a lone prompt and halves a lane's
+  // products; measured, a token takes as long: its cost is the sums across lanes, the hand-over and
+  // the waits, not the products.)
   int P = 1;
   while (P * SCAN_ROWS < D) P <<= 1;
   const int cols = 256 / P, Dp = P * SCAN_ROWS;
-  const int CH = min(Dp <= 128 ? 16 : (Dp <= 256 ? 8 : 4), 8 * P);     // 8 values a thread of each kind a chunk
-  const size_t lds = (size_t)CH * ((mode == SCAN_LSTM ? 2 : 3) * Dp + cols + 2) * sizeof(float);
+  const int CH = min(min(16, 2048 / Dp), 8 * P);       // 8 values a thread of each kind a chunk
+  const size_t lds = 2 * (size_t)CH * ((mode == SCAN_LSTM ? 2 : 3) * Dp + 2 * cols + 4) * sizeof(float);   // two halves
   const MatrixScan a{src, src_stride, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, gates, gate_stride,
                      i_col, f_col, cap, state, state_stride, cu_q, positions, slots, write, out};
   const dim3 grid(S, H, (Dv + cols - 1) / cols);
-  if (mode == SCAN_DECAY) matrix_scan_kernel<SCAN_DECAY><<<grid, 256, lds, stream>>>(a, P, CH);
-  else if (mode == SCAN_DELTA) matrix_scan_kernel<SCAN_DELTA><<<grid, 256, lds, stream>>>(a, P, CH);
-  else matrix_scan_kernel<SCAN_LSTM><<<grid, 256, lds, stream>>>(a, P, CH);
+  if (mode == SCAN_DECAY) matrix_scan_kernel<SCAN_DECAY, SCAN_ROWS><<<grid, 512, lds, stream>>>(a, P, CH);
+  else if (mode == SCAN_DELTA) matrix_scan_kernel<SCAN_DELTA, SCAN_ROWS><<<grid, 512, lds, stream>>>(a, P, CH);
+  else matrix_scan_kernel<SCAN_LSTM, SCAN_ROWS><<<grid, 512, lds, stream>>>(a, P, CH);
   return sl_launch_status();
 }
 
