@@ -213,18 +213,26 @@ class VekanexConfig:
                 raise ConfigError(f"config.json: {where} must be an object")
             owner = entry.get("weights_of")
             if owner is not None:
-                owner = read_key(entry, "weights_of", kind=int)
-                if not 0 <= owner < len(entries) or owner == i or entries[owner].get("weights_of") is not None:
-                    raise ConfigError(f"config.json: {where}: weights_of must name another layer that "
-                                      "has tensors of its own")
+                # the layer whose tensors these are, through any layers that borrow them in turn
+                owner, seen = read_key(entry, "weights_of", kind=int), {i}
+                while True:
+                    if not 0 <= owner < len(entries) or owner in seen or not isinstance(entries[owner], dict):
+                        raise ConfigError(f"config.json: {where}: weights_of must lead to another layer "
+                                          "that has tensors of its own")
+                    if entries[owner].get("weights_of") is None:
+                        break
+                    seen.add(owner)
+                    owner = read_key(entries[owner], "weights_of", kind=int)
+                # what the entry leaves out it takes from the owner's
+                entry = dict(entries[owner], **{k: v for k, v in entry.items() if k != "weights_of"})
             kind = read_key(entry, "type", kind=str)
             prefix = f"l{i if owner is None else owner}.mix."
             mixer = _read_mixer(kind, _section(entry, "mixer", where), prefix, shapes, where)
             layers.append(VekanexLayer(kind, mixer, _read_mlp(entry.get("mlp"), where), owner))
         out = cls(width=read_key(cfg, "width", kind=int), vocab=read_key(cfg, "vocab", kind=int),
                   norm_eps=read_key(norm, "eps", kind=float),
-                  residual_mult=read_key(cfg, "residual_mult", kind=float),
-                  logit_softcap=read_key(cfg, "logit_softcap", kind=float), layers=layers,
+                  residual_mult=read_key(cfg, "residual_mult", 1.0, kind=float),
+                  logit_softcap=read_key(cfg, "logit_softcap", 0.0, kind=float), layers=layers,
                   architecture=str(cfg.get("architecture") or "Vekanex"),
                   dtype=str(cfg.get("torch_dtype") or "bfloat16"), path=path, raw=dict(cfg))
         out.validate()
@@ -233,8 +241,8 @@ class VekanexConfig:
     def validate(self) -> None:
         if self.width < 1 or self.vocab < 1 or not self.norm_eps > 0:
             raise ConfigError("config.json: width and vocab must be positive, norm.eps > 0")
-        if not self.logit_softcap > 0:
-            raise ConfigError("config.json: logit_softcap must be positive")
+        if self.logit_softcap < 0:                # 0 (or no key): the logits stay as they are
+            raise ConfigError("config.json: logit_softcap must not be negative")
         for i, l in enumerate(self.layers):
             if l.weights_of is not None:
                 o = self.layers[l.weights_of]

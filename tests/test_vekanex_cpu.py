@@ -48,7 +48,7 @@ def test_config_round_trip_and_declared_tensors(tmp_path, which):
 
 def test_missing_and_impossible_keys_name_themselves():
     base = MODELS["A"]
-    for path, text in ((("residual_mult",), "residual_mult"), (("logit_softcap",), "logit_softcap"),
+    for path, text in ((("width",), "width"), (("norm",), "norm"),
                        (("layers", 1, "mixer", "gate_cap"), "gate_cap"),
                        (("layers", 2, "mixer", "tau"), "tau"),
                        (("layers", 0, "mixer", "left", "rot"), "rot"),
@@ -77,9 +77,25 @@ def test_missing_and_impossible_keys_name_themselves():
     with pytest.raises(ConfigError, match="another layer"):
         VekanexConfig.from_hf(cfg)
     cfg = copy.deepcopy(base)
+    cfg["layers"][3]["weights_of"], cfg["layers"][0]["weights_of"] = 0, 3      # a ring: nobody has tensors
+    with pytest.raises(ConfigError, match="weights_of"):
+        VekanexConfig.from_hf(cfg)
+    cfg = copy.deepcopy(base)
     cfg["layers"][1]["type"] = "rnn"
     with pytest.raises(ConfigError, match="mlstm, gla, parallel"):
         VekanexConfig.from_hf(cfg)
+
+
+def test_borrowed_layers_and_keys_that_may_be_left_out():
+    cfg = copy.deepcopy(MODELS["A"])
+    cfg["layers"][4] = {"weights_of": 3}               # borrows from a borrower, and says nothing else
+    del cfg["logit_softcap"], cfg["residual_mult"]
+    got = VekanexConfig.from_hf(cfg)
+    assert got.layers[4].weights_of == 0 and got.layers[4].mixer == got.layers[0].mixer
+    assert got.layers[4].mlp == got.layers[0].mlp and got.layers[4].kind == "parallel"
+    assert got.logit_softcap == 0.0 and got.residual_mult == 1.0
+    spec = build_model_spec(got)
+    assert [c.layer for c in spec.run] == [0, 1, 2, 0, 0] and spec.head[1].softcap is None
 
 
 def test_cache_needs_and_run_list():
