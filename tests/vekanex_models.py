@@ -80,13 +80,14 @@ def _c():
 def _d():
     # a convolution of one tap (no inputs kept); head counts that are no powers of two; channel
     # counts that are no multiples of four; two rotated channels; more experts than a wavefront has
-    # lanes; a layer that borrows from one behind it
+    # lanes; a layer that borrows from one behind it; two attentions whose pages differ in size
     layers = [
         parallel((5, 5, 12, 20, 0.4, 100.0, 2), (5, 1, 20, 12, 1, 2, 3), 0.3, 1.1, moe(70, 9, 8)),
         gla(5, 20, 12, 1.0, 2, moe(2, 2, 12, 4)),
         mlstm(5, 12, 20, 3.0, moe(2, 1, 12, 4)),
+        parallel((2, 1, 16, 8, 0.25, 7.0, 16), (3, 3, 8, 8, 5, 1, 1), 1.0, -0.5, None),
     ]
-    return config(40, 97, 1e-4, 0.25, 5.0, [dict(again(layers, 2), weights_of=3)] + layers[:2] + [layers[2]])
+    return config(40, 97, 1e-4, 0.25, 5.0, [dict(again(layers, 2), weights_of=3)] + layers[:2] + layers[2:])
 
 
 MODELS = {"A": _a(), "B": _b(), "C": _c(), "D": _d()}
