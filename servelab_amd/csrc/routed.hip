@@ -138,7 +138,22 @@ struct Grouped {
   int N, K;
   act_t* out_act;            // gated: [rows][N]
   float* out_f32;            // plain: [rows][N]
+  int max_tiles, col_blocks; // the matrix-core kernels' launch: max_tiles x col_blocks workgroups in a row
 };
+
+// Which (row tile, column block) a workgroup of a one-dimensional launch takes.  Workgroups go to the
+// chip's eight dies in turn (number % 8), and each die has an L2 of its own: a die gets a contiguous
+// run of the list ordered by column block, then row tile, so the row tiles of one expert, which read
+// the same columns of the same matrices, run on one die at about the same time and the matrices
+// come from memory once.
+__device__ __forceinline__ bool grouped_place(const Grouped& a, int& tile, int& cb) {
+  const int total = a.max_tiles * a.col_blocks, run = (total + 7) / 8;
+  const int m = (blockIdx.x & 7) * run + (blockIdx.x >> 3);
+  if ((int)(blockIdx.x >> 3) >= run || m >= total) return false;
+  cb = m / a.max_tiles;
+  tile = m - cb * a.max_tiles;
+  return true;
+}
 
 // 256 threads: thread (row = tid / 16, lane16 = tid % 16) owns columns lane16 + 16 u, u < 4, of a
 // 16 x 64 tile.  x and W go through LDS in chunks of 32 values of k; sums are float.
@@ -214,10 +229,12 @@ template <int NT, int NU, bool GATED, int WR, int WC>
 __global__ __launch_bounds__(64 * WR * WC) void grouped_product_mfma_kernel(const Grouped a) {
   // WR x WC wavefronts a workgroup: WR along the rows of the row tile, WC along the columns; those
   // that read the same rows of x or of W find them in the CU's cache after the first has asked
-  const int* tl = a.tiles + 3 * blockIdx.x;
+  int tile, cb;
+  if (!grouped_place(a, tile, cb)) return;
+  const int* tl = a.tiles + 3 * tile;
   const int wave = threadIdx.x / 64, wr = wave % WR, wc = wave / WR;
   const int rows = min(16 * NT, tl[2] - 16 * NT * wr);
-  const int n0 = (blockIdx.y * WC + wc) * 16 * NU;
+  const int n0 = (cb * WC + wc) * 16 * NU;
   if (rows <= 0 || n0 >= a.N) return;
   const int e = tl[0], row0 = tl[1] + 16 * NT * wr;
   const int lane = threadIdx.x & 63, i = lane & 15, gq = lane >> 4;
@@ -287,6 +304,7 @@ __global__ __launch_bounds__(64 * WR * WC) void grouped_product_mfma_kernel(cons
     }
   }
 }
+
 #endif
 
 extern "C" const char* sl_grouped_product(const void* x, const int* order, int top, const void* w, const int* tiles,
@@ -295,25 +313,24 @@ extern "C" const char* sl_grouped_product(const void* x, const int* order, int t
   SL_CHECK(max_tiles >= 0 && N > 0 && K > 0 && top >= 1, "grouped_product: sizes must be positive");
   SL_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "grouped_product: row tiles hold 16, 64 or 128 rows");
   if (max_tiles == 0) return nullptr;
-  const Grouped a{(const act_t*)x, order, top, (const act_t*)w, w_tiled, tiles, tile_rows / RT_ROWS, N, K,
-                  gated ? (act_t*)out : nullptr, gated ? nullptr : (float*)out};
+  Grouped a{(const act_t*)x, order, top, (const act_t*)w, w_tiled, tiles, tile_rows / RT_ROWS, N, K,
+            gated ? (act_t*)out : nullptr, gated ? nullptr : (float*)out, max_tiles, 1};
 #if !defined(SL_F32)
-#if defined(SL_F32)
-  SL_CHECK(!w_tiled, "grouped_product: tiled matrices are for bfloat16");
-#endif
   if (K % 32 == 0 && N % 16 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0) {
-    if (tile_rows == 128) {                             // two wavefronts along the rows, two along the columns
-      const dim3 grid(max_tiles, (N + 127) / 128);
-      if (gated) grouped_product_mfma_kernel<4, 4, true, 2, 2><<<grid, 256, 0, stream>>>(a);
-      else grouped_product_mfma_kernel<4, 4, false, 2, 2><<<grid, 256, 0, stream>>>(a);
+    // (a one-dimensional launch of max_tiles x col_blocks workgroups, rounded up to the eight dies)
+    auto blocks = [&](int cols) {
+      a.col_blocks = (N + cols - 1) / cols;
+      return dim3(8 * (unsigned)((max_tiles * a.col_blocks + 7) / 8));
+    };
+    if (tile_rows == 128) {                      // two wavefronts along the rows, two along the columns
+      if (gated) grouped_product_mfma_kernel<4, 4, true, 2, 2><<<blocks(128), 256, 0, stream>>>(a);
+      else grouped_product_mfma_kernel<4, 4, false, 2, 2><<<blocks(128), 256, 0, stream>>>(a);
     } else if (tile_rows == 64) {
-      const dim3 grid(max_tiles, (N + 255) / 256);
-      if (gated) grouped_product_mfma_kernel<4, 4, true, 1, 4><<<grid, 256, 0, stream>>>(a);
-      else grouped_product_mfma_kernel<4, 4, false, 1, 4><<<grid, 256, 0, stream>>>(a);
+      if (gated) grouped_product_mfma_kernel<4, 4, true, 1, 4><<<blocks(256), 256, 0, stream>>>(a);
+      else grouped_product_mfma_kernel<4, 4, false, 1, 4><<<blocks(256), 256, 0, stream>>>(a);
     } else {
-      const dim3 grid(max_tiles, (N + 63) / 64);
-      if (gated) grouped_product_mfma_kernel<1, 4, true, 1, 1><<<grid, 64, 0, stream>>>(a);
-      else grouped_product_mfma_kernel<1, 4, false, 1, 1><<<grid, 64, 0, stream>>>(a);
+      if (gated) grouped_product_mfma_kernel<1, 4, true, 1, 1><<<blocks(64), 64, 0, stream>>>(a);
+      else grouped_product_mfma_kernel<1, 4, false, 1, 1><<<blocks(64), 64, 0, stream>>>(a);
     }
     return sl_launch_status();
   }

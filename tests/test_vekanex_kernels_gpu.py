@@ -224,7 +224,8 @@ def test_route_tokens_sorts_the_pairs_by_expert(T, E, top):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,E,top,ff,K", [(1, 5, 2, 24, 64), (9, 12, 4, 64, 72), (150, 8, 3, 40, 96), (20, 3, 3, 8, 200),
-                                          (9, 6, 2, 48, 64), (150, 8, 3, 80, 96), (400, 6, 2, 160, 128)])
+                                          (9, 6, 2, 48, 64), (150, 8, 3, 80, 96), (400, 6, 2, 160, 128),
+                                          (700, 4, 2, 192, 128), (900, 3, 3, 64, 320)])
 def test_routed_experts(dtype, T, E, top, ff, K):
     hip, emu = tables(dtype)
     g = torch.Generator().manual_seed(11)
