@@ -26,36 +26,57 @@ __device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-
 // ------------------------------------------------------------------ low-rank expansion
 // out[t][c] = f(sum_r buf[t][col + r] W2[c][r] + bias[c]);  mode 0: z, 1: logsigmoid(z) / divisor,
 // 2: -exp(rates[c / per_head]) * softplus(z)
-__global__ void lowrank_expand_kernel(const float* __restrict__ buf, int stride, int col, int rank,
-                                      const float* __restrict__ w2, const float* __restrict__ bias, int C,
-                                      int mode, float divisor, const float* __restrict__ rates, int per_head,
-                                      float* __restrict__ out) {
-  extern __shared__ float low[];
-  const size_t t = blockIdx.x;
-  for (int r = threadIdx.x; r < rank; r += blockDim.x) low[r] = buf[t * stride + col + r];
+// A workgroup takes LOW_TOKENS tokens by 256 channels: a thread reads its channel's row of W2 once
+// for all of them.
+#define LOW_TOKENS 8
+__global__ __launch_bounds__(256) void lowrank_expand_kernel(const float* __restrict__ buf, int stride, int col,
+                                                             int rank, const float* __restrict__ w2,
+                                                             const float* __restrict__ bias, int T, int C, int mode,
+                                                             float divisor, const float* __restrict__ rates,
+                                                             int per_head, float* __restrict__ out) {
+  extern __shared__ float low[];                       // [LOW_TOKENS][rank]
+  const size_t t0 = (size_t)blockIdx.x * LOW_TOKENS;
+  const int nt = min(LOW_TOKENS, T - (int)t0);
+  for (int i = threadIdx.x; i < LOW_TOKENS * rank; i += blockDim.x) {
+    const int tt = i / rank, r = i - tt * rank;
+    low[i] = tt < nt ? buf[(t0 + tt) * stride + col + r] : 0.f;
+  }
   __syncthreads();
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
   const float* w = w2 + (size_t)c * rank;
-  float z = 0.f;
-  for (int r = 0; r < rank; ++r) z += low[r] * w[r];
-  if (bias != nullptr) z += bias[c];
-  if (mode == 1) z = logsigmoidf_(z) / divisor;
-  else if (mode == 2) z = -expf(rates[c / per_head]) * softplusf_(z);
-  out[t * C + c] = z;
+  float z[LOW_TOKENS];
+#pragma unroll
+  for (int tt = 0; tt < LOW_TOKENS; ++tt) z[tt] = 0.f;
+  for (int r = 0; r < rank; ++r) {
+    const float wr = w[r];
+#pragma unroll
+    for (int tt = 0; tt < LOW_TOKENS; ++tt) z[tt] += low[tt * rank + r] * wr;
+  }
+  const float b = bias != nullptr ? bias[c] : 0.f;
+  const float rate = mode == 2 ? -expf(rates[c / per_head]) : 0.f;
+#pragma unroll
+  for (int tt = 0; tt < LOW_TOKENS; ++tt) {
+    if (tt >= nt) break;
+    float v = z[tt] + b;
+    if (mode == 1) v = logsigmoidf_(v) / divisor;
+    else if (mode == 2) v = rate * softplusf_(v);
+    out[(t0 + tt) * C + c] = v;
+  }
 }
 
 extern "C" const char* sl_lowrank_expand(const float* buf, int stride, int col, int rank, const float* w2,
                                          const float* bias, int T, int C, int mode, float divisor,
                                          const float* rates, int heads, float* out, hipStream_t stream) {
-  SL_CHECK(T >= 0 && C > 0 && rank > 0 && rank <= 8192, "lowrank_expand: sizes must be positive, rank <= 8192");
+  SL_CHECK(T >= 0 && C > 0 && rank > 0 && rank <= 1024, "lowrank_expand: sizes must be positive, rank <= 1024");
   SL_CHECK(col >= 0 && col + rank <= stride, "lowrank_expand: the columns do not fit the rows");
   SL_CHECK(mode >= 0 && mode <= 2 && heads > 0 && C % heads == 0, "lowrank_expand: unknown mode or heads");
   SL_CHECK(mode != 2 || rates != nullptr, "lowrank_expand: rates are missing");
   SL_CHECK(mode != 1 || divisor > 0.f, "lowrank_expand: the divisor must be positive");
   if (T == 0) return nullptr;
-  lowrank_expand_kernel<<<dim3(T, (C + 255) / 256), 256, rank * sizeof(float), stream>>>(
-      buf, stride, col, rank, w2, bias, C, mode, divisor, rates, C / heads, out);
+  lowrank_expand_kernel<<<dim3((T + LOW_TOKENS - 1) / LOW_TOKENS, (C + 255) / 256), 256,
+                          LOW_TOKENS * rank * sizeof(float), stream>>>(
+      buf, stride, col, rank, w2, bias, T, C, mode, divisor, rates, C / heads, out);
   return sl_launch_status();
 }
 
