@@ -175,7 +175,7 @@ def test_the_program_replays_a_trace(tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B"])
+@pytest.mark.parametrize("which", ["A", "B", "E"])
 def test_greedy_generation_through_the_entry_point(tmp_path, which, dtype):
     cfg = MODELS[which]
     folder, weights = write_folder(tmp_path, cfg, seed=15, tag=which)

@@ -90,7 +90,17 @@ def _d():
     return config(40, 97, 1e-4, 0.25, 5.0, [dict(again(layers, 2), weights_of=3)] + layers[:2] + layers[2:])
 
 
-MODELS = {"A": _a(), "B": _b(), "C": _c(), "D": _d()}
+def _e():
+    # no attention at all: the engine holds states and not one page; the decay's projection as wide
+    # as a head's key; a feed-forward of one expert that every token takes
+    layers = [
+        gla(2, 16, 16, 6.0, 16, moe(1, 1, 32)),
+        mlstm(2, 16, 8, 8.0, moe(6, 3, 16, 16)),
+    ]
+    return config(48, 200, 1e-5, 1.5, 8.0, layers + [again(layers, 0)])
+
+
+MODELS = {"A": _a(), "B": _b(), "C": _c(), "D": _d(), "E": _e()}
 
 
 def tensor_shapes(cfg):
