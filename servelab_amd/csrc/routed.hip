@@ -305,6 +305,119 @@ __global__ __launch_bounds__(64 * WR * WC) void grouped_product_mfma_kernel(cons
   }
 }
 
+
+// Row tiles of 128 rows with the rows of x staged in LDS: a workgroup of four wavefronts takes a row
+// tile by 64 NU columns; every wavefront owns all 128 rows by 16 NU columns (of the gate and of the
+// up matrix in the gated form).  The tile's rows of x come 64 values of k at a time into one of two
+// halves of LDS (a thread brings four 16-byte pieces, asked for one step ahead); a row's eight pieces
+// are stored at piece ^ (row / 2 % 8), so that the 16 lanes of a fragment read, and the 16 of a
+// write, take every bank once.  W comes straight from memory in the tiled layout, a k-step ahead: no
+// two wavefronts of the workgroup read the same piece of it, and the CU's cache delivers a third of
+// what the unstaged kernel asks of it.  Two workgroups a CU: one computes while the other waits.
+template <int NU, bool GATED>
+__global__ __launch_bounds__(256, 2) void grouped_product_staged_kernel(const Grouped a) {
+  constexpr int NT = 8, MATS = GATED ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) __bf16 stage[2][128 * 64];
+  int tile, cb;
+  if (!grouped_place(a, tile, cb)) return;
+  const int* tl = a.tiles + 3 * tile;
+  const int rows = min(128, tl[2]);
+  if (rows <= 0) return;                                // (the whole workgroup: no barrier is left waiting)
+  const int e = tl[0], row0 = tl[1];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x & 63, i = lane & 15, gq = lane >> 4;
+  const int n0 = (cb * 4 + wave) * 16 * NU;
+  const size_t n_w = GATED ? 2 * (size_t)a.N : (size_t)a.N;
+  const __bf16* we = a.w + (size_t)e * n_w * a.K;
+  const size_t up = (size_t)a.N * a.K;
+  const __bf16* wp[NU];
+#pragma unroll
+  for (int u = 0; u < NU; ++u)
+    wp[u] = we + (size_t)(min(n0 + 16 * u, a.N - 16) / 16) * (a.K / 32) * 512 + lane * 8;
+  // what this thread brings: piece threadIdx % 8 of rows threadIdx / 8 + 32 j
+  const int piece = threadIdx.x & 7, rbase = threadIdx.x >> 3;
+  const __bf16* xsrc[4];
+  int xat[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = rbase + 32 * j, rr = row0 + min(r, rows - 1);
+    const size_t src = a.order != nullptr ? (size_t)(a.order[rr] / a.top) : (size_t)rr;
+    xsrc[j] = a.x + src * a.K + 8 * piece;
+    xat[j] = r * 64 + 8 * (piece ^ ((r >> 1) & 7));
+  }
+  const int fsw = (i >> 1) & 7;                         // (16 v + i) / 2 % 8
+  rt_f32x4 acc[NT][NU * MATS];
+#pragma unroll
+  for (int v = 0; v < NT; ++v)
+#pragma unroll
+    for (int u = 0; u < NU * MATS; ++u) acc[v][u] = rt_f32x4{0.f, 0.f, 0.f, 0.f};
+  rt_bf16x8 xr[4], wcur[NU * MATS], wnext[NU * MATS];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) xr[j] = *(const rt_bf16x8*)(xsrc[j]);
+#pragma unroll
+  for (int u = 0; u < NU; ++u) {
+    wcur[u] = *(const rt_bf16x8*)(wp[u]);
+    if (GATED) wcur[NU + u] = *(const rt_bf16x8*)(wp[u] + up);
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) *(rt_bf16x8*)(&stage[0][xat[j]]) = xr[j];
+  __syncthreads();
+  const int steps = a.K / 64;
+  for (int s = 0; s < steps; ++s) {
+    if (s + 1 < steps) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xr[j] = *(const rt_bf16x8*)(xsrc[j] + 64 * (s + 1));
+    }
+    const __bf16* buf = stage[s & 1] + i * 64;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int kstep = 2 * s + h;
+      if (kstep + 1 < 2 * steps) {
+        const size_t kw = (size_t)(kstep + 1) * 512;
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+          wnext[u] = *(const rt_bf16x8*)(wp[u] + kw);
+          if (GATED) wnext[NU + u] = *(const rt_bf16x8*)(wp[u] + up + kw);
+        }
+      }
+      const int fo = 8 * ((4 * h + gq) ^ fsw);
+#pragma unroll
+      for (int v = 0; v < NT; ++v) {
+        const rt_bf16x8 b = *(const rt_bf16x8*)(buf + v * 16 * 64 + fo);
+#pragma unroll
+        for (int u = 0; u < NU * MATS; ++u)
+          acc[v][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wcur[u], b, acc[v][u], 0, 0, 0);
+      }
+#pragma unroll
+      for (int u = 0; u < NU * MATS; ++u) wcur[u] = wnext[u];
+    }
+    if (s + 1 < steps) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) *(rt_bf16x8*)(&stage[(s + 1) & 1][xat[j]]) = xr[j];
+    }
+    __syncthreads();
+  }
+  // this lane holds columns n0 + 16 u + 4 gq .. + 3 of rows 16 v + i
+#pragma unroll
+  for (int v = 0; v < NT; ++v) {
+    if (16 * v + i >= rows) continue;
+    const size_t at = (size_t)(row0 + 16 * v + i) * a.N + n0 + 4 * gq;
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+      if (n0 + 16 * u >= a.N) continue;
+      if (GATED) {
+        rt_bf16x4 r;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const float g = acc[v][u][c];
+          r[c] = (__bf16)(g / (1.f + expf(-g)) * acc[v][NU + u][c]);
+        }
+        *(rt_bf16x4*)(a.out_act + at + 16 * u) = r;
+      } else {
+        *(rt_f32x4*)(a.out_f32 + at + 16 * u) = acc[v][u];
+      }
+    }
+  }
+}
 #endif
 
 extern "C" const char* sl_grouped_product(const void* x, const int* order, int top, const void* w, const int* tiles,
@@ -322,7 +435,10 @@ extern "C" const char* sl_grouped_product(const void* x, const int* order, int t
       a.col_blocks = (N + cols - 1) / cols;
       return dim3(8 * (unsigned)((max_tiles * a.col_blocks + 7) / 8));
     };
-    if (tile_rows == 128) {                      // two wavefronts along the rows, two along the columns
+    if (tile_rows == 128 && w_tiled && K % 64 == 0) {   // the tile's rows of x staged in LDS
+      if (gated) grouped_product_staged_kernel<2, true><<<blocks(128), 256, 0, stream>>>(a);
+      else grouped_product_staged_kernel<4, false><<<blocks(256), 256, 0, stream>>>(a);
+    } else if (tile_rows == 128) {                      // two wavefronts along the rows, two along the columns
       if (gated) grouped_product_mfma_kernel<4, 4, true, 2, 2><<<blocks(128), 256, 0, stream>>>(a);
       else grouped_product_mfma_kernel<4, 4, false, 2, 2><<<blocks(128), 256, 0, stream>>>(a);
     } else if (tile_rows == 64) {
