@@ -246,6 +246,10 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
   const int tid = threadIdx.x & 255;
   const int Dp = P * ROWS, cols = 256 / P;
   const int lgDp = __ffs(Dp) - 1, lgCols = __ffs(cols) - 1;
+  // The matrix LSTM's normaliser n is one more column of S whose value channel is always 1: the last
+  // column group of every block carries it (every block the same one) and leaves max(|n . q|, e^-m) +
+  // 1e-6 where the others leave their read-outs; these are divided by it when they leave LDS.
+  const int vcols = MODE == SCAN_LSTM ? cols - 1 : cols;
   const int half = CH * ((MODE == SCAN_LSTM ? 2 : 3) * Dp + 2 * cols + 4);
   const int oq = 0, ok = CH * Dp, oa = 2 * CH * Dp;          // [CH][Dp] each (no decays for the matrix LSTM)
   const int ov = MODE == SCAN_LSTM ? oa : oa + CH * Dp;       // [CH][cols]
@@ -283,8 +287,9 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
           }
         }
         if (idx < nt * cols) {
-          const int tt = idx >> lgCols, cc = slice * cols + (idx & (cols - 1));
-          if (cc < a.Dv) pv[e] = a.src[(size_t)(t0 + tt) * a.src_stride + a.v_col + h * a.Dv + cc];
+          const int tt = idx >> lgCols, cl = idx & (cols - 1), cc = slice * vcols + cl;
+          if (cl >= vcols) pv[e] = 1.f;
+          else if (cc < a.Dv) pv[e] = a.src[(size_t)(t0 + tt) * a.src_stride + a.v_col + h * a.Dv + cc];
         }
       }
       if (MODE != SCAN_DECAY && tid < 64 && tid < nt) {
@@ -299,8 +304,11 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
       const float* so = lds + (c & 1) * half + oo;
       const int tf = t0 - 2 * CH, nf = min(CH, last - tf);
       for (int idx = tid; idx < nf * cols; idx += 256) {
-        const int jj = slice * cols + (idx & (cols - 1));
-        if (jj < a.Dv) a.out[((size_t)(tf + (idx >> lgCols)) * a.H + h) * a.Dv + jj] = so[idx];
+        const int tt = idx >> lgCols, cl = idx & (cols - 1), jj = slice * vcols + cl;
+        if (cl >= vcols || jj >= a.Dv) continue;
+        float o = so[idx];
+        if (MODE == SCAN_LSTM) o = o / so[tt * cols + cols - 1];
+        a.out[((size_t)(tf + tt) * a.H + h) * a.Dv + jj] = o;
       }
     };
     ask(first, min(CH, last - first));
@@ -359,10 +367,11 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
   }
 
   const int p = tid & (P - 1), cl = tid >> (__ffs(P) - 1);
-  const int j = slice * cols + cl;
-  const bool live = j < a.Dv;
-  float* col = slot + ((size_t)h * a.Dv + (live ? j : 0)) * a.D;
-  float S[ROWS], n[ROWS];
+  const bool is_n = MODE == SCAN_LSTM && cl == cols - 1;
+  const int j = slice * vcols + cl;
+  const bool live = is_n || j < a.Dv;
+  float* col = is_n ? nrow : slot + ((size_t)h * a.Dv + (live ? j : 0)) * a.D;
+  float S[ROWS];
   const int r0 = p * ROWS;
   // (a lane's values of a column are 16-byte pieces where the slot's place allows it)
   const bool whole = live && r0 + ROWS <= a.D && ((uintptr_t)(col + r0) % 16) == 0;
@@ -378,7 +387,6 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
   for (int i = 0; i < ROWS; ++i) {
     const int r = r0 + i;
     if (!(whole && !fresh)) S[i] = (!fresh && live && r < a.D) ? col[r] : 0.f;
-    n[i] = (MODE == SCAN_LSTM && !fresh && r < a.D) ? nrow[r] : 0.f;
   }
   __syncthreads();                        // chunk 0 is in LDS
   for (int t0 = first, c = 0; t0 < last; t0 += CH, ++c) {
@@ -409,7 +417,6 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
         }
       }
       const float v = sv[tt * cols + cl];
-      float o, floor_ = 0.f;
       float part[ROWS];
       if (MODE == SCAN_DECAY) {
 #pragma unroll
@@ -432,27 +439,21 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
           part[i] = S[i] * q[i];
         }
       } else {
-        const float keep = sg[tt * 4], add = sg[tt * 4 + 1];
-        floor_ = sg[tt * 4 + 2];
-        float npart[ROWS];
+        const float keep = sg[tt * 4], av = sg[tt * 4 + 1] * v;     // (v is 1 in the column that carries n)
 #pragma unroll
         for (int i = 0; i < ROWS; ++i) {
-          const float ak = add * k[i];
-          S[i] = keep * S[i] + ak * v;
-          n[i] = keep * n[i] + ak;
+          S[i] = keep * S[i] + k[i] * av;
           part[i] = S[i] * q[i];
-          npart[i] = n[i] * q[i];
         }
-        const float nq = group_sum(rows_sum<ROWS>(npart), P);
-        floor_ = fmaxf(fabsf(nq), floor_) + 1e-6f;
       }
-      o = group_sum(rows_sum<ROWS>(part), P);
-      if (MODE == SCAN_LSTM) o = o / floor_;
+      float o = group_sum(rows_sum<ROWS>(part), P);
+      // (the column that carries n leaves the divisor of its token's read-outs)
+      if (MODE == SCAN_LSTM && is_n) o = fmaxf(fabsf(o), sg[tt * 4 + 2]) + 1e-6f;
       if (p == 0) so[tt * cols + cl] = o;
     }
     __syncthreads();                      // chunk c + 1 is in LDS, chunk c's half is free
   }
-  if (a.write) {
+  if (a.write && (!is_n || slice == 0)) {             // (every slice carries the same n: the first writes it)
     if (whole) {
 #pragma unroll
       for (int u = 0; u < ROWS / 4; ++u) {
@@ -466,7 +467,6 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
     for (int i = 0; i < ROWS; ++i) {
       const int r = r0 + i;
       if (!whole && live && r < a.D) col[r] = S[i];
-      if (MODE == SCAN_LSTM && slice == 0 && cl == 0 && r < a.D) nrow[r] = n[i];
     }
   }
 }
@@ -499,7 +499,8 @@ extern "C" const char* sl_matrix_scan(int mode, const float* src, int src_stride
   const size_t lds = 2 * (size_t)CH * ((mode == SCAN_LSTM ? 2 : 3) * Dp + 2 * cols + 4) * sizeof(float);   // two halves
   const MatrixScan a{src, src_stride, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, gates, gate_stride,
                      i_col, f_col, cap, state, state_stride, cu_q, positions, slots, write, out};
-  const dim3 grid(S, H, (Dv + cols - 1) / cols);
+  const int vcols = mode == SCAN_LSTM ? cols - 1 : cols;       // (the matrix LSTM's last column group carries n)
+  const dim3 grid(S, H, (Dv + vcols - 1) / vcols);
   if (mode == SCAN_DECAY) matrix_scan_kernel<SCAN_DECAY, SCAN_ROWS><<<grid, 512, lds, stream>>>(a, P, CH);
   else if (mode == SCAN_DELTA) matrix_scan_kernel<SCAN_DELTA, SCAN_ROWS><<<grid, 512, lds, stream>>>(a, P, CH);
   else matrix_scan_kernel<SCAN_LSTM, SCAN_ROWS><<<grid, 512, lds, stream>>>(a, P, CH);
