@@ -27,8 +27,8 @@ __device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-
 // out[t][c] = f(sum_r buf[t][col + r] W2[c][r] + bias[c]);  mode 0: z, 1: logsigmoid(z) / divisor,
 // 2: -exp(rates[c / per_head]) * softplus(z)
 // A workgroup takes LOW_TOKENS tokens by 256 channels: a thread reads its channel's row of W2 once
-// for all of them.
-#define LOW_TOKENS 8
+// for all of them (8 tokens in a prompt's portion; 1 in a step of few tokens, which needs the blocks).
+template <int LOW_TOKENS>
 __global__ __launch_bounds__(256) void lowrank_expand_kernel(const float* __restrict__ buf, int stride, int col,
                                                              int rank, const float* __restrict__ w2,
                                                              const float* __restrict__ bias, int T, int C, int mode,
@@ -74,9 +74,12 @@ extern "C" const char* sl_lowrank_expand(const float* buf, int stride, int col, 
   SL_CHECK(mode != 2 || rates != nullptr, "lowrank_expand: rates are missing");
   SL_CHECK(mode != 1 || divisor > 0.f, "lowrank_expand: the divisor must be positive");
   if (T == 0) return nullptr;
-  lowrank_expand_kernel<<<dim3((T + LOW_TOKENS - 1) / LOW_TOKENS, (C + 255) / 256), 256,
-                          LOW_TOKENS * rank * sizeof(float), stream>>>(
-      buf, stride, col, rank, w2, bias, T, C, mode, divisor, rates, C / heads, out);
+  if (T >= 32)
+    lowrank_expand_kernel<8><<<dim3((T + 7) / 8, (C + 255) / 256), 256, 8 * rank * sizeof(float), stream>>>(
+        buf, stride, col, rank, w2, bias, T, C, mode, divisor, rates, C / heads, out);
+  else
+    lowrank_expand_kernel<1><<<dim3(T, (C + 255) / 256), 256, rank * sizeof(float), stream>>>(
+        buf, stride, col, rank, w2, bias, T, C, mode, divisor, rates, C / heads, out);
   return sl_launch_status();
 }
 
